@@ -1,0 +1,267 @@
+"""Benchmark of the W4A16 hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep] [--no-cpu]
+
+Default workload (the line the driver records): the decode sweep's M = 1 column,
+"llama31_8b_decode_layer_m1": one step = the four W4A16 GEMVs of a Llama-3.1-8B
+decoder layer at M = 1 (fused qkv 4096->6144, o_proj 4096->4096, fused gate_up
+4096->28672, down_proj 14336->4096; group 128, fp16 scales, fp16 activations).
+Inputs are synthetic (codes U{0..15}, scales U[0.004,0.02], x ~ N(0,1), seed 1234) and
+resident in HBM before the timed region.  Successive steps use different weight
+copies whose total size exceeds the 256 MB last-level cache, so the weights come
+from HBM, not from cache.  Steps are replayed as HIP graphs (one per weight copy)
+so that launch overhead is the GPU's, not Python's.
+
+value = algorithmic bytes per step / time per step  (GB/s), algorithmic bytes of a
+linear = K N / 2 + (K/128) N 2 + M K 2 + M N 2.
+
+--sweep additionally prints (stderr) and writes (gpurun_out/bench_sweep.json) the
+per-shape tables: decode M in {1,2,4,8}, prefill M in {256,1024,4096}, the pruned
+Llama shapes with the fused 128-block rotation, the Mamba2 shapes, the embedding
+gather and the standalone transform.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
+LLC_BYTES = 256 << 20
+
+LLAMA_DECODE = [("qkv", 4096, 6144), ("o_proj", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
+PRUNED = [("q_pruned", 4096, 3584, 0), ("o_pruned", 3456, 4096, 0), ("gate_up_pruned", 4096, 24320, 0),
+          ("down_pruned_had128", 12160, 4096, 128)]
+MAMBA = [("mamba_in_proj", 4096, 18688, 0), ("mamba_out_proj_had8192", 8192, 4096, 8192)]
+
+
+def linear_bytes(m, k, n):
+    return k * n // 2 + (k // 128) * n * 2 + m * k * 2 + m * n * 2
+
+
+def linear_flops(m, k, n):
+    return 2 * m * k * n
+
+
+# --------------------------------------------------------------------------------------
+def make_weights(k, n, dev, gen):
+    """Random packed tensors directly on the device: uniformly random 32-bit words are
+    uniformly random int4 codes in every nibble of the packed layout."""
+    import torch
+    b = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 16, 2 * n), dtype=torch.int64, device=dev, generator=gen).to(torch.int32)
+    s = (torch.rand((k // 128, n), device=dev, generator=gen) * 0.016 + 0.004).to(torch.float16)
+    return b, s
+
+
+class Layer:
+    """One linear shape with `copies` independent weight sets."""
+
+    def __init__(self, name, k, n, m, copies, dev, gen, had_block=0):
+        import torch
+        self.name, self.k, self.n, self.m, self.had_block = name, k, n, m, had_block
+        self.weights = [make_weights(k, n, dev, gen) for _ in range(copies)]
+        self.x = torch.randn((m, k), device=dev, generator=gen).to(torch.float16)
+        self.ws = torch.zeros((n // 64) * 16, dtype=torch.int32, device=dev)
+
+    def run(self, i):
+        from uniql_amd import ops
+        b, s = self.weights[i % len(self.weights)]
+        if self.had_block:
+            return ops.w4a16_gemm_ex(self.x, b, s, self.ws, self.m, self.n, self.k, had_block=self.had_block,
+                                     had_scale=self.had_block ** -0.5)
+        return ops.w4a16o16_gemm(self.x, b, s, self.ws, self.m, self.n, self.k, False, -1, -1, -1, 16)
+
+
+def time_graphs(run_step, n_variants, steps, warmup):
+    """Captures run_step(i) for i < n_variants as HIP graphs, replays them round-robin and
+    returns seconds per step measured with events on the launch stream."""
+    import torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for i in range(n_variants):
+            run_step(i)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graphs, keep = [], []
+    for i in range(n_variants):
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            keep.append(run_step(i))
+        graphs.append(g)
+    for i in range(warmup):
+        graphs[i % n_variants].replay()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()
+    for i in range(steps):
+        graphs[i % n_variants].replay()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return start.elapsed_time(stop) * 1e-3 / steps, wall / steps
+
+
+def copies_for(bytes_per_copy):
+    return max(2, int(np.ceil(1.5 * LLC_BYTES / bytes_per_copy)) + 1)
+
+
+# --------------------------------------------------------------------------------------
+def cpu_baseline(sample_reps=3):
+    """The reference's CPU meaning of the layer (unpack -> un-permute -> (q-8)*s -> fp32 matmul),
+    restated by the oracle, timed on this host for the o_proj shape at M = 1."""
+    import torch
+
+    from oracle import uniql_oracle as O
+    k = n = 4096
+    rng = np.random.default_rng(1234)
+    packed = rng.integers(-2 ** 31, 2 ** 31 - 1, size=(k // 16, 2 * n), dtype=np.int64).astype(np.int32)
+    s_perm = rng.uniform(0.004, 0.02, size=(k // 128, n)).astype(np.float16)
+    x = rng.standard_normal((1, k)).astype(np.float16)
+    times = []
+    for _ in range(sample_reps + 1):
+        t0 = time.perf_counter()
+        w = O.dequant_packed(packed, s_perm, k, n)
+        y = O.gemm_fp32(x, w)
+        times.append(time.perf_counter() - t0)
+    best = float(np.median(times[1:]))
+    t1 = time.perf_counter()
+    for _ in range(10):
+        y = O.gemm_fp32(x, w)
+    matmul_only = (time.perf_counter() - t1) / 10
+    del y
+    return {
+        "value": round(linear_bytes(1, k, n) / best / 1e9, 4), "unit": "GB/s", "cores": torch.get_num_threads(),
+        "kind": "port",
+        "sample": f"o_proj 4096x4096 M=1, unpack+unpermute+dequant+fp32 matmul, median of {sample_reps} runs "
+                  f"({best * 1e3:.1f} ms each; matmul alone on pre-dequantised fp32 weights {matmul_only * 1e3:.2f} ms); "
+                  f"host has {os.cpu_count()} cpus",
+    }
+
+
+# --------------------------------------------------------------------------------------
+def sweep(dev, gen, out_path):
+    import torch
+
+    from uniql_amd import ops
+    rows = []
+
+    def bench_linear(name, k, n, m, had_block=0, steps=200):
+        per = linear_bytes(m, k, n)
+        copies = copies_for(k * n // 2) if m <= 64 else 2
+        layer = Layer(name, k, n, m, copies, dev, gen, had_block)
+        sec, _ = time_graphs(lambda i: layer.run(i), copies, steps, 20)
+        row = dict(op=name, m=m, k=k, n=n, had_block=had_block, us=sec * 1e6, gbs=per / sec / 1e9,
+                   hbm_frac=per / sec / 1e9 / HBM_PEAK_GBS, tflops=linear_flops(m, k, n) / sec / 1e12,
+                   mfma_frac=linear_flops(m, k, n) / sec / 1e12 / MFMA_F16_PEAK_TFLOPS)
+        rows.append(row)
+        print("%-24s M=%-5d K=%-6d N=%-6d %9.2f us %8.1f GB/s (%5.1f%% HBM) %8.1f TFLOP/s (%5.1f%% MFMA)" % (
+            name, m, k, n, row["us"], row["gbs"], 100 * row["hbm_frac"], row["tflops"], 100 * row["mfma_frac"]),
+            file=sys.stderr, flush=True)
+        del layer
+        torch.cuda.empty_cache()
+
+    for m in (1, 2, 4, 8):
+        for name, k, n in LLAMA_DECODE:
+            bench_linear(name, k, n, m)
+    for m in (256, 1024, 4096):
+        for name, k, n in LLAMA_DECODE:
+            bench_linear(name, k, n, m, steps=20)
+    for m in (1, 1024):
+        for name, k, n, hb in PRUNED + MAMBA:
+            bench_linear(name, k, (n + 255) // 256 * 256, m, hb, steps=200 if m == 1 else 20)
+
+    # embedding gather: V = 256000, D = 4096, 2048 ids
+    v, d, t = 256000, 4096, 2048
+    table = torch.randint(-2 ** 31, 2 ** 31 - 1, (v, d // 8), dtype=torch.int64, device=dev, generator=gen).to(torch.int32)
+    scales = (torch.rand(v, device=dev, generator=gen) * 0.016 + 0.004).to(torch.float16)
+    idsets = [torch.randint(0, v, (t,), device=dev, generator=gen) for _ in range(8)]
+    sec, _ = time_graphs(lambda i: ops.w4a16_embedding_lookup(idsets[i], table, scales), 8, 200, 20)
+    per = t * (d // 2 + 2 + 8 + 2 * d)
+    rows.append(dict(op="embedding_256000x4096", tokens=t, us=sec * 1e6, gbs=per / sec / 1e9,
+                     hbm_frac=per / sec / 1e9 / HBM_PEAK_GBS))
+    print("embedding 256000x4096, 2048 ids: %.2f us %.1f GB/s (%.1f%% HBM)" % (
+        sec * 1e6, per / sec / 1e9, 100 * per / sec / 1e9 / HBM_PEAK_GBS), file=sys.stderr, flush=True)
+    del table
+
+    for rows_x, dim, block in ((1, 8192, 8192), (1024, 8192, 8192), (1024, 12160 + 128, 128)):
+        xs = [torch.randn((rows_x, dim), device=dev, generator=gen).to(torch.float16) for _ in range(4)]
+        sec, _ = time_graphs(lambda i: ops.hadamard_blockwise(xs[i], block ** -0.5, block), 4, 200, 20)
+        per = rows_x * dim * 4
+        rows.append(dict(op=f"fwht_block{block}", rows=rows_x, dim=dim, us=sec * 1e6, gbs=per / sec / 1e9))
+        print("fwht rows=%d dim=%d block=%d: %.2f us %.1f GB/s" % (rows_x, dim, block, sec * 1e6, per / sec / 1e9),
+              file=sys.stderr, flush=True)
+
+    os.makedirs(os.path.dirname(out_path), exist_ok=True)
+    with open(out_path, "w") as f:
+        json.dump(rows, f, indent=1)
+
+
+# --------------------------------------------------------------------------------------
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=40)
+    ap.add_argument("--sweep", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev).manual_seed(1234)
+
+    m = 1
+    step_bytes = sum(linear_bytes(m, k, n) for _, k, n in LLAMA_DECODE)
+    weight_bytes = sum(k * n // 2 for _, k, n in LLAMA_DECODE)
+    copies = copies_for(weight_bytes)
+    layers = [Layer(name, k, n, m, copies, dev, gen) for name, k, n in LLAMA_DECODE]
+
+    def run_step(i):
+        return [layer.run(i) for layer in layers]
+
+    sec_per_step, wall_per_step = time_graphs(run_step, copies, args.steps, args.warmup)
+    launches = len(layers)
+    gbs = step_bytes / sec_per_step / 1e9
+    kernel_us = sec_per_step / launches * 1e6
+    result = {
+        "metric": "W4A16 GEMV GB/s at M=1 (Llama-3.1-8B decoder-layer linears)", "value": round(gbs, 2),
+        "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(sec_per_step * 1e3, 6), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16 (int4 weights, fp32 accumulate)", "data": "synthetic",
+        "config": {"workload": "llama31_8b_decode_layer_m1", "linears": [f"{n_}:{k}x{n}" for n_, k, n in LLAMA_DECODE],
+                   "m": m, "group_size": 128, "weight_copies_rotated": copies, "launch": "hip_graph",
+                   "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "wall_ms_per_step": round(wall_per_step * 1e3, 6)},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
+                     "kernel": "w4a16_stream_kernel<1,false>", "launches_per_step": launches,
+                     "avg_launch_us": round(kernel_us, 3), "bytes_per_launch": step_bytes // launches},
+    }
+    del layers
+    torch.cuda.empty_cache()
+    if args.sweep:
+        sweep(dev, gen, os.path.join(ROOT, "gpurun_out", "bench_sweep.json"))
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,120 @@
+/*
+ * uniql_amd.h - C ABI of the MI355X (gfx950) W4A16 kernels.
+ *
+ * Plain pointers and sizes only.  All pointers named "device" are HIP device
+ * addresses on the current device.  `stream` is a hipStream_t passed as
+ * void* (NULL = the default stream).  No entry point synchronises the stream
+ * or frees memory; every call only enqueues kernels, so all of them can be
+ * recorded into a HIP graph.  Return value: 0 on success, a negative
+ * UNIQL_E_* code otherwise (nothing was launched then).
+ *
+ * Paths in the comments are files of the reference (enyac-group/UniQL).
+ */
+#ifndef UNIQL_AMD_H
+#define UNIQL_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define UNIQL_ABI_VERSION 1
+
+enum {
+    UNIQL_OK = 0,
+    UNIQL_E_NULL = -1,        /* a required pointer is NULL                        */
+    UNIQL_E_SHAPE = -2,       /* m/n/k/groups violate the layout's divisibility    */
+    UNIQL_E_ALIGN = -3,       /* a pointer or leading dimension is not 16-byte aligned */
+    UNIQL_E_WORKSPACE = -4,   /* workspace or scratch too small                    */
+    UNIQL_E_UNSUPPORTED = -5, /* valid request this build does not implement       */
+    UNIQL_E_LAUNCH = -6       /* the HIP runtime rejected a launch                 */
+};
+
+/* flags of uniql_w4a16_gemm */
+enum {
+    UNIQL_F_OUT_F32 = 1 << 0,      /* D is float32 [m, n] instead of fp16 (test hook: the value before the final rounding) */
+    UNIQL_F_FORCE_SKINNY = 1 << 1, /* use the weight-streaming kernel whatever m is */
+    UNIQL_F_FORCE_TILED = 1 << 2,  /* use the prefill (LDS + MFMA tile) kernel whatever m is */
+    UNIQL_F_TRANSPOSE_OUT = 1 << 3 /* reference's output_transpose; rejected with UNIQL_E_UNSUPPORTED */
+    /* bits 8..15: units-per-wave override for the skinny kernel (0 = heuristic); tuning hook */
+};
+
+int uniql_abi_version(void);
+const char* uniql_status_string(int code);
+
+/*
+ * D[m, n] = A[m, k] . dequant(B)[k, n],  fp16 in, fp32 accumulate, fp16 out.
+ * Replaces quant_linear_cuda.w4a16o16_gemm (csrc/linear/quant_linear.cpp:6-24,
+ * host wrapper csrc/linear/marlin_gemm_kernel.cuh:991-1052).
+ *
+ *   A          device, fp16 [m, k] row-major, row stride lda elements (lda >= k, lda % 8 == 0)
+ *   B          device, int32 [k/16, 2 n]: the packed layout written by
+ *              quantize/quantize_helpers.py:66-84 with the table of :144-165
+ *   S          device, fp16 [groups, n], permuted by quantize_helpers.py:168-180;
+ *              groups == k/128 (group-128 scales) or groups == 1 (one scale per column)
+ *   D          device, fp16 [m, n] row-major (float32 with UNIQL_F_OUT_F32)
+ *   workspace  device, int32 [workspace_len] >= n/128 entries, all zero on entry;
+ *              zero again when the kernels have finished (the module's
+ *              `workspace` buffer, quantize/quant_linear_layers.py:33-35)
+ *   scratch    device, at least uniql_w4a16_gemm_scratch_bytes(m, n, k) bytes,
+ *              contents irrelevant (replaces the reference's per-call `C`
+ *              allocation, marlin_gemm_kernel.cuh:1018); may be NULL if that size is 0
+ *   had_block  0: none.  Otherwise the activations are rotated first,
+ *              A <- fp16(A . H_had_block * had_scale) on consecutive
+ *              had_block-wide pieces of each row: 128 is fused into the
+ *              streaming kernel's prologue, any other power of two (<= 32768,
+ *              dividing k) runs the transform kernel into scratch first.
+ *   k % 128 == 0, n % 128 == 0 (the module pads n to 256).
+ */
+size_t uniql_w4a16_gemm_scratch_bytes(int m, int n, int k, int had_block);
+
+int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, void* D,
+                     int32_t* workspace, int64_t workspace_len,
+                     void* scratch, size_t scratch_bytes,
+                     int m, int n, int k, int groups,
+                     int had_block, float had_scale,
+                     unsigned flags, void* stream);
+
+/*
+ * W[k, n] fp16 = fp16_rn((code - 8) * scale), natural (un-permuted) order.
+ * The value csrc/linear/marlin_gemm_kernel.cuh:118-146 builds in registers and
+ * quantize/quantize_helpers.py:118 calls w_ref.  Also writes the raw codes
+ * (uint8 [k, n]) when `codes` is not NULL: the inverse of
+ * quantize_helpers.py:303-328 on the device.
+ */
+int uniql_w4a16_dequant(const void* B, const void* S, void* W, uint8_t* codes,
+                        int n, int k, int groups, void* stream);
+
+/*
+ * out[t, :] = fp16_rn((code - 8) * scales[ids[t]]) for t < ntokens.
+ * Replaces quant_embedding_cuda.w4a16_embedding_lookup
+ * (csrc/embedding/quant_embedding_kernel.cuh:80-166).
+ *   ids     device, int64 [ntokens]; each id must be in [0, vocab)
+ *   weight  device, int32 [vocab, dim/8], packing of quantize/quant_embedding_layers.py:33-43
+ *   scales  device, fp16 [vocab]
+ *   out     device, fp16 [ntokens, dim];  dim % 8 == 0
+ */
+int uniql_w4_embedding_lookup(const int64_t* ids, int64_t ntokens,
+                              const void* weight, const void* scales, void* out,
+                              int64_t vocab, int dim, void* stream);
+
+/*
+ * y[r, :] = round((x[r, :] . H) * scale), H = Sylvester Hadamard matrix applied
+ * to consecutive `block`-wide pieces of each row (block == dim: the whole row);
+ * butterflies in fp32, one rounding to the element type at the end.
+ * Replaces fast_hadamard_transform_cuda.fast_hadamard_transform(x, scale) as
+ * called by quantize/hadamard_helpers.py:22-48 (power-of-two case).
+ *   x, y   device, [rows, dim] contiguous, element type `dtype` (UNIQL_DT_*); y may equal x
+ *   block  power of two, 2 <= block <= 32768, dim % block == 0
+ */
+enum { UNIQL_DT_F16 = 0, UNIQL_DT_BF16 = 1, UNIQL_DT_F32 = 2 };
+
+int uniql_fwht(const void* x, void* y, int64_t rows, int dim, int block,
+               float scale, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* UNIQL_AMD_H */

@@ -1,0 +1,386 @@
+"""CPU oracle for UniQL's W4A16 hot path.  TEST INFRASTRUCTURE ONLY.
+
+This file restates, in numpy / CPU torch, what the reference computes on the
+path  pack -> (GPU) dequant + matmul,  the per-row int4 embedding lookup and
+the Walsh-Hadamard rotation.  It is the checker that tests/, the smoke test
+and the `cpu_baseline` leg of bench.py compare the HIP kernels against.  It is
+never imported by the `uniql_amd` package: the product path has no CPU
+fallback.
+
+Every function names the reference lines it follows (paths relative to the
+reference checkout).
+
+Pinning status (what proves each function right, besides reading):
+  * weight permutation / pack / unpack ....... golden vectors produced by the
+    reference's own quantize_helpers + an independent closed-form index map
+    + bijection / round-trip properties
+  * scale permutations ....................... golden vectors + closed form
+  * group-128 quantiser (code selection) ..... golden vectors
+  * dequant fp16_rn((q-8)*s) ................. closed form, exhaustive in tests
+  * dequant + matmul ......................... brute-force loops on tiny shapes
+  * embedding quantise/pack/lookup ........... hand-computed tiny cases +
+    brute-force; the reference module cannot be imported without its compiled
+    extension, so `embedding_quantize`'s code selection at exact rounding ties
+    is "parity unpinned" beyond those cases
+  * power-of-two Hadamard .................... scipy.linalg.hadamard, involution,
+    Parseval.  The 12N/20N/28N/40N variants need base matrices that live in an
+    un-vendored third-party package (Dao-AILab fast-hadamard-transform, commit
+    unknown): they are not restated here and are "parity unpinned".
+"""
+from __future__ import annotations
+
+import math
+
+import numpy as np
+import torch
+
+TILE = 16          # quantize_helpers.py:13  (GPTQ_MARLIN_TILE)
+PACK = 8           # quantize_helpers.py:31-34 with num_bits = 4
+GROUP = 128        # quantize_helpers.py:16   (only 128 and -1 are supported)
+MIN_THREAD_N = 64  # quantize_helpers.py:10
+MAX_PARALLEL = 16  # quantize_helpers.py:12
+
+
+# --------------------------------------------------------------------------
+# a1: weight permutation table and the nibble packer
+# --------------------------------------------------------------------------
+def weight_perm_table() -> np.ndarray:
+    """1024-entry gather table.  Follows quantize_helpers.py:144-165."""
+    out = []
+    for lane in range(32):
+        eight = []
+        col = lane // 4
+        for block in (0, 1):
+            for row in (2 * (lane % 4), 2 * (lane % 4) + 1,
+                        2 * (lane % 4 + 4), 2 * (lane % 4 + 4) + 1):
+                eight.append(16 * row + col + 8 * block)
+        for j in range(4):
+            out.extend(p + 256 * j for p in eight)
+    table = np.asarray(out, dtype=np.int64)
+    interleave = np.array([0, 2, 4, 6, 1, 3, 5, 7])
+    return table.reshape(-1, 8)[:, interleave].ravel()
+
+
+def scale_perm_tables():
+    """(grouped, per-channel) scale gather tables.  quantize_helpers.py:53-62."""
+    grouped = []
+    for i in range(8):
+        grouped.extend(i + 8 * j for j in range(8))
+    single = []
+    for i in range(4):
+        single.extend(2 * i + j for j in (0, 1, 8, 9, 16, 17, 24, 25))
+    return np.asarray(grouped), np.asarray(single)
+
+
+def tile_and_permute(q: np.ndarray) -> np.ndarray:
+    """[K, N] codes -> [K/16, 16 N] in kernel order.  quantize_helpers.py:37-50."""
+    k, n = q.shape
+    assert k % TILE == 0 and n % TILE == 0
+    t = q.reshape(k // TILE, TILE, n // TILE, TILE).transpose(0, 2, 1, 3)
+    t = t.reshape(k // TILE, n * TILE)
+    perm = weight_perm_table()
+    return t.reshape(-1, perm.size)[:, perm].reshape(t.shape)
+
+
+def pack_weights(q: np.ndarray) -> np.ndarray:
+    """[K, N] codes in 0..15 -> int32 [K/16, 2 N].  quantize_helpers.py:66-84."""
+    t = tile_and_permute(np.asarray(q)).astype(np.uint32)
+    packed = np.zeros((t.shape[0], t.shape[1] // PACK), dtype=np.uint32)
+    for i in range(PACK):
+        packed |= t[:, i::PACK] << np.uint32(4 * i)
+    return packed.view(np.int32)
+
+
+def unpack_weights(packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    """int32 [K/16, 2 N] -> [K, N] codes.  quantize_helpers.py:278-328."""
+    u = np.ascontiguousarray(packed).view(np.uint32)
+    assert u.shape == (size_k // TILE, size_n * TILE // PACK)
+    t = np.zeros((u.shape[0], u.shape[1] * PACK), dtype=np.uint32)
+    for i in range(PACK):
+        t[:, i::PACK] = (u >> np.uint32(4 * i)) & np.uint32(0xF)
+    perm = weight_perm_table()
+    inv = np.empty_like(perm)
+    inv[perm] = np.arange(perm.size)
+    t = t.reshape(-1, perm.size)[:, inv].reshape(size_k // TILE, size_n * TILE)
+    t = t.reshape(size_k // TILE, size_n // TILE, TILE, TILE).transpose(0, 2, 1, 3)
+    return np.ascontiguousarray(t.reshape(size_k, size_n)).astype(np.int32)
+
+
+# --------------------------------------------------------------------------
+# a2: scale permutation
+# --------------------------------------------------------------------------
+def _grouped(size_k: int, group_size: int) -> bool:
+    # quantize_helpers.py:171 / :259
+    return group_size < size_k and group_size != -1
+
+
+def permute_scales(scale: np.ndarray, size_k: int, size_n: int, group_size: int) -> np.ndarray:
+    """quantize_helpers.py:168-180."""
+    grouped, single = scale_perm_tables()
+    tab = grouped if _grouped(size_k, group_size) else single
+    return np.ascontiguousarray(scale.reshape(-1, tab.size)[:, tab].reshape(-1, size_n))
+
+
+def unpermute_scales(scale: np.ndarray, size_k: int, size_n: int, group_size: int) -> np.ndarray:
+    """quantize_helpers.py:244-275."""
+    grouped, single = scale_perm_tables()
+    tab = grouped if _grouped(size_k, group_size) else single
+    inv = np.argsort(tab)
+    return np.ascontiguousarray(scale.reshape(-1, tab.size)[:, inv].reshape(-1, size_n))
+
+
+# --------------------------------------------------------------------------
+# a3: the group-128 symmetric quantiser (fp16 arithmetic on the CPU)
+# --------------------------------------------------------------------------
+@torch.no_grad()
+def fake_quantize_grouped(w: torch.Tensor, group_size: int = GROUP):
+    """fp16 [K, N] -> (w_ref fp16 [Kp, N], codes int32 [Kp, N], scale fp16 [Kp/g, N]).
+
+    Follows quantize_helpers.py:87-121 (the per-group branch): the arithmetic
+    is done by CPU torch in the tensor's own dtype, as the reference does.
+    """
+    size_k, size_n = w.shape
+    assert group_size < size_k
+    pad_k = (-size_k) % group_size
+    if pad_k:
+        w = torch.nn.functional.pad(w, (0, 0, 0, pad_k))
+    g = w.reshape(-1, group_size, size_n)
+    scale = g.abs().max(dim=1, keepdim=True)[0]
+    scale *= 2 / 15
+    q = torch.round(g / scale).int()      # NaN (0/0) becomes 0 in .int()
+    q += 8
+    q = torch.clamp(q, 0, 15)
+    w_ref = (q - 8) * scale
+    return (w_ref.reshape(-1, size_n).contiguous(),
+            q.reshape(-1, size_n).contiguous(),
+            scale.reshape(-1, size_n).contiguous())
+
+
+@torch.no_grad()
+def requantize_with_scales(w: torch.Tensor, scale: torch.Tensor, group_size: int = GROUP):
+    """Codes for weights that were already fake-quantised with the given
+    group scales (the GPTQ branch).  quantize_helpers.py:205-218."""
+    size_k, size_n = w.shape
+    pad_k = (-size_k) % group_size
+    if pad_k:
+        w = torch.nn.functional.pad(w, (0, 0, 0, pad_k))
+    w_ref = w.clone()
+    g = w.reshape(-1, group_size, size_n)
+    q = ((g / scale.unsqueeze(1)) + 8).round().int()
+    q = torch.clamp(q, 0, 15).reshape(size_k + pad_k, size_n).contiguous()
+    return w_ref, q, scale
+
+
+@torch.no_grad()
+def w4a16_quantize(w: torch.Tensor, group_size: int = GROUP, scale: torch.Tensor | None = None,
+                   pad_out: int = 0):
+    """fp16 [K, N] -> (w_ref, packed int32 [Kp/16, 2 Np], permuted scale fp16 [Kp/g, Np]).
+
+    Follows quantize_helpers.py:183-241 for the group-128 case.  The
+    per-channel case (in_features <= 128) packs signed codes unmasked in the
+    reference (quantize_helpers.py:123-135 with :75-80), which no supported
+    model reaches; it is not restated.
+    """
+    size_k, size_n = w.shape
+    assert group_size == GROUP and group_size < size_k
+    if scale is None:
+        w_ref, q, scale = fake_quantize_grouped(w, group_size)
+    else:
+        w_ref, q, scale = requantize_with_scales(w, scale, group_size)
+    if pad_out:
+        w_ref = torch.nn.functional.pad(w_ref, (0, pad_out))
+        q = torch.nn.functional.pad(q, (0, pad_out))
+        scale = torch.nn.functional.pad(scale, (0, pad_out))
+    kp, np_ = w_ref.shape
+    packed = torch.from_numpy(pack_weights(q.numpy()))
+    s_perm = torch.from_numpy(permute_scales(scale.numpy(), kp, np_, group_size))
+    return w_ref, packed, s_perm
+
+
+# --------------------------------------------------------------------------
+# a9: dequantisation, and the reference's CPU meaning of the linear layer
+# --------------------------------------------------------------------------
+def dequant_codes(q: np.ndarray, scale: np.ndarray, group_size: int = GROUP) -> np.ndarray:
+    """codes [K, N], natural-order scale fp16 [K/g or 1, N] -> fp16 [K, N].
+
+    w = fp16_rn(float(q - 8) * float(s)):  marlin_gemm_kernel.cuh:118-146 (the
+    magic-number conversion yields q-8 exactly, then one fp16 multiply), equal
+    to the CPU expression at quantize_helpers.py:118 and
+    modeling/modeling_helpers.py:632-640.
+    """
+    k, n = q.shape
+    s = np.asarray(scale, dtype=np.float16)
+    if s.shape[0] == 1:
+        s_full = np.broadcast_to(s, (k, n))
+    else:
+        s_full = np.repeat(s, group_size, axis=0)
+    prod = (q.astype(np.float32) - 8.0) * s_full.astype(np.float32)   # exact in fp32
+    return prod.astype(np.float16)
+
+
+def dequant_packed(packed: np.ndarray, scale_perm: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    """Packed kernel-layout tensors -> dequantised fp16 [K, N]."""
+    groups = scale_perm.shape[0]
+    group_size = size_k // groups if groups > 1 else -1   # marlin_gemm_kernel.cuh:1008
+    q = unpack_weights(packed, size_k, size_n)
+    s = unpermute_scales(np.asarray(scale_perm), size_k, size_n,
+                         group_size if group_size != -1 else size_k)
+    return dequant_codes(q, s, group_size if group_size != -1 else size_k)
+
+
+def gemm_fp32(x: np.ndarray, w_deq: np.ndarray) -> np.ndarray:
+    """fp16 [M, K] x fp16 [K, N] -> float32 [M, N], accumulated in (at least)
+    fp32.  The textbook product the kernel must match
+    (marlin_gemm_kernel.cuh:443-462: fp16 operands, fp32 accumulate)."""
+    xt = torch.from_numpy(np.ascontiguousarray(x)).to(torch.float32)
+    wt = torch.from_numpy(np.ascontiguousarray(w_deq)).to(torch.float32)
+    return torch.matmul(xt, wt).numpy()
+
+
+def gemm_fp64(x: np.ndarray, w_deq: np.ndarray) -> np.ndarray:
+    """Same product accumulated in float64 (the exact value up to 1e-13)."""
+    return np.asarray(x, dtype=np.float64) @ np.asarray(w_deq, dtype=np.float64)
+
+
+def linear_forward(x: np.ndarray, packed: np.ndarray, scale_perm: np.ndarray, *,
+                   in_features: int, out_features: int, bias: np.ndarray | None = None,
+                   exact: bool = False) -> np.ndarray:
+    """What W4A16B16O16Linear.forward returns, before the final fp16 rounding.
+
+    quant_linear_layers.py:91-116: flatten, zero-pad K, product, drop padded
+    output columns, restore leading shape, add bias.
+    Returns float32 (or float64 if exact) of shape (*x.shape[:-1], out_features).
+    """
+    size_k = packed.shape[0] * TILE
+    size_n = packed.shape[1] * PACK // TILE
+    lead = x.shape[:-1]
+    x2 = np.asarray(x, dtype=np.float16).reshape(-1, x.shape[-1])
+    assert x2.shape[1] == in_features
+    if size_k != in_features:
+        x2 = np.pad(x2, ((0, 0), (0, size_k - in_features)))
+    w = dequant_packed(packed, scale_perm, size_k, size_n)
+    y = gemm_fp64(x2, w) if exact else gemm_fp32(x2, w)
+    y = y[:, :out_features].reshape(*lead, out_features)
+    if bias is not None:
+        y = y + np.asarray(bias, dtype=y.dtype)
+    return y
+
+
+# --------------------------------------------------------------------------
+# a10/a11: int4 embedding with one scale per vocabulary row
+# --------------------------------------------------------------------------
+EMB_INTERLEAVE = np.array([0, 2, 4, 6, 1, 3, 5, 7])   # quant_embedding_layers.py:33
+
+
+@torch.no_grad()
+def embedding_quantize(w: torch.Tensor):
+    """[V, D] float -> (packed int32 [V, D/8], scales fp16 [V]).
+
+    quant_embedding_layers.py:35-46: arithmetic in the weight's own dtype.
+    """
+    v, d = w.shape
+    scales = w.abs().amax(dim=-1, keepdim=True) / 8
+    q = torch.round((w / scales) + 8).clamp(0, 15)
+    q = q.to(torch.int32).numpy().astype(np.uint32)
+    q = q.reshape(v, -1, 8)[:, :, EMB_INTERLEAVE].reshape(v, -1)
+    packed = np.zeros((v, d // PACK), dtype=np.uint32)
+    for i in range(PACK):
+        packed |= (q[:, i::PACK] & np.uint32(0xF)) << np.uint32(4 * i)
+    return packed.view(np.int32), scales.flatten().to(torch.float16).numpy()
+
+
+def embedding_unpack(packed: np.ndarray) -> np.ndarray:
+    """int32 [V, D/8] -> codes [V, D] in natural element order (inverse of the
+    interleaved packing at quant_embedding_layers.py:39-43)."""
+    u = np.ascontiguousarray(packed).view(np.uint32)
+    v, words = u.shape
+    codes = np.zeros((v, words, 8), dtype=np.int32)
+    for i in range(PACK):
+        codes[:, :, EMB_INTERLEAVE[i]] = ((u >> np.uint32(4 * i)) & np.uint32(0xF)).astype(np.int32)
+    return codes.reshape(v, words * 8)
+
+
+def embedding_lookup(ids: np.ndarray, packed: np.ndarray, scales: np.ndarray) -> np.ndarray:
+    """out[..., :] = fp16_rn((code - 8) * scale[id]).
+    quant_embedding_kernel.cuh:47-76 (conversion exact, one fp16 multiply) and
+    :80-114 (one scale per token row, natural output order)."""
+    ids = np.asarray(ids)
+    rows = embedding_unpack(packed[ids.reshape(-1)])
+    s = np.asarray(scales, dtype=np.float16)[ids.reshape(-1)].astype(np.float32)[:, None]
+    out = ((rows.astype(np.float32) - 8.0) * s).astype(np.float16)
+    return out.reshape(*ids.shape, rows.shape[1])
+
+
+# --------------------------------------------------------------------------
+# a12/a13: Walsh-Hadamard rotation
+# --------------------------------------------------------------------------
+def is_pow2(n: int) -> bool:
+    return n > 0 and (n & (n - 1)) == 0     # hadamard_helpers.py:4-5
+
+
+def had_variant(dim: int):
+    """(base N, scale) chosen for a width.  hadamard_helpers.py:18-36."""
+    scale = 1.0 / math.sqrt(dim)
+    for base in (40, 28, 20, 12):
+        if dim % base == 0 and is_pow2(dim // base):
+            return base, scale
+    assert is_pow2(dim), f"Invalid dim: {dim}. dim must be a power of 2."
+    return 2, scale
+
+
+def fwht(x: np.ndarray, scale: float, block: int | None = None,
+         acc=np.float32) -> np.ndarray:
+    """y = (x . H_block) * scale along the last axis, H the Sylvester
+    (natural-order) Hadamard matrix, applied independently to consecutive
+    `block`-wide pieces (block = whole width by default).  Internal arithmetic
+    in `acc`, result rounded to x's dtype: the contract of
+    fast_hadamard_transform(x, scale) as called at hadamard_helpers.py:35,45
+    and quant_hadamard_layers.py:18.
+    """
+    dim = x.shape[-1]
+    block = dim if block is None else block
+    assert is_pow2(block) and dim % block == 0
+    y = np.asarray(x).astype(acc).reshape(-1, dim // block, block).copy()
+    h = 1
+    while h < block:
+        y = y.reshape(y.shape[0], y.shape[1], block // (2 * h), 2, h)
+        a = y[:, :, :, 0, :].copy()
+        b = y[:, :, :, 1, :].copy()
+        y[:, :, :, 0, :] = a + b
+        y[:, :, :, 1, :] = a - b
+        y = y.reshape(y.shape[0], y.shape[1], block)
+        h *= 2
+    y = y * acc(scale)
+    return y.reshape(x.shape).astype(x.dtype)
+
+
+def hadamard_module_forward(x: np.ndarray, dim: int) -> np.ndarray:
+    """Hadamard(dim).forward(x).  quant_hadamard_layers.py:5-21."""
+    base, scale = had_variant(dim)
+    assert base == 2, "non power-of-two variants are not restated (parity unpinned)"
+    return fwht(x, scale)
+
+
+def hadlinear_fused_weight(w: np.ndarray, input_transform: bool = True,
+                           output_transform: bool = False) -> np.ndarray:
+    """HadLinear.fuse_hadamard on W [Dout, Din].  quant_linear_layers.py:159-167."""
+    w = np.asarray(w)
+    if input_transform:
+        w = fwht(w, 1.0 / math.sqrt(w.shape[1]))
+    if output_transform:
+        w = np.ascontiguousarray(fwht(np.ascontiguousarray(w.T), 1.0 / math.sqrt(w.shape[0])).T)
+    return w
+
+
+# --------------------------------------------------------------------------
+# module buffer geometry (a4)
+# --------------------------------------------------------------------------
+def linear_geometry(in_features: int, out_features: int, group_size: int = GROUP):
+    """Padded sizes and buffer shapes.  quant_linear_layers.py:13-48."""
+    pad_out = (-out_features) % 256
+    pad_in = (-in_features) % group_size
+    size_n, size_k = out_features + pad_out, in_features + pad_in
+    return dict(size_n=size_n, size_k=size_k, pad_in=pad_in, pad_out=pad_out,
+                workspace=(size_n // MIN_THREAD_N) * MAX_PARALLEL,
+                weight=(size_k // 16, size_n * 16 // 8),
+                scale=(size_k // group_size, size_n))

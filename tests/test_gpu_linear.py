@@ -1,0 +1,166 @@
+"""GPU parity of the W4A16 linear path, through the C ABI (ops -> ctypes -> HIP)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import uniql_oracle as O
+from tests.helpers import (check_layer_output, make_linear_problem, reference_product, to_gpu,
+                           workspace_for)
+
+pytestmark = pytest.mark.gpu
+
+
+def run_gemm(p, dev, **kw):
+    from uniql_amd import ops
+    x, b, s = to_gpu(p, dev)
+    ws = workspace_for(p["n"], dev)
+    y = ops.w4a16_gemm_ex(x, b, s, ws, p["m"], p["n"], p["k"], **kw)
+    torch.cuda.synchronize()
+    assert int(ws.abs().sum()) == 0, "workspace must be zero again after the call"
+    return y.cpu().numpy()
+
+
+# ------------------------------------------------------------------ bit-exact layer
+@pytest.mark.parametrize("k,n", [(128, 128), (256, 256), (512, 384), (4096, 4096)])
+def test_dequant_and_codes_bit_exact(gpu, k, n):
+    from uniql_amd import ops
+    p = make_linear_problem(1, k, n, seed=k + n)
+    _, b, s = to_gpu(p, gpu)
+    w, codes = ops.w4a16_dequant(b, s, n, k, want_codes=True)
+    assert np.array_equal(codes.cpu().numpy().astype(np.int32), p["q"])
+    want = O.dequant_codes(p["q"], p["s"])
+    assert np.array_equal(w.cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
+def test_dequant_every_code_times_every_scale(gpu):
+    """16 codes x all 63488 finite fp16 scales (both signs, subnormals included)."""
+    from uniql_amd import ops
+    bits = np.arange(0x10000, dtype=np.uint32).astype(np.uint16)
+    finite = bits[(bits & 0x7C00) != 0x7C00]
+    n = 63488 // 128 * 128
+    assert finite.size == 63488 and n == 63488
+    s = finite.view(np.float16).reshape(1, n)
+    k = 128
+    q = np.tile(np.arange(16, dtype=np.int32)[:, None], (k // 16, n))
+    packed = torch.from_numpy(O.pack_weights(q)).to(gpu)
+    s_perm = torch.from_numpy(O.permute_scales(s, k, n, k)).to(gpu)
+    w = ops.w4a16_dequant(packed, s_perm, n, k).cpu().numpy()
+    want = O.dequant_codes(q, s, k)
+    assert np.array_equal(w.view(np.uint16), want.view(np.uint16))
+
+
+def test_dequant_golden_case(gpu, golden):
+    from uniql_amd import ops
+    b = torch.from_numpy(golden["A_packed"]).to(gpu)
+    s = torch.from_numpy(golden["A_scale"]).to(gpu)
+    w, codes = ops.w4a16_dequant(b, s, 256, 256, want_codes=True)
+    assert np.array_equal(codes.cpu().numpy(), golden["A_codes"])
+    assert np.array_equal(w.cpu().numpy().view(np.uint16), golden["A_w_ref"].view(np.uint16))
+
+
+# ------------------------------------------------------------------ decode shapes
+@pytest.mark.parametrize("m", [1, 2, 3, 4, 8, 16])
+@pytest.mark.parametrize("k,n", [(128, 128), (256, 256), (640, 384), (4096, 4096)])
+def test_stream_kernel_small_m(gpu, m, k, n):
+    p = make_linear_problem(m, k, n, seed=100 * m + k // 128 + n)
+    ref = reference_product(p, exact=True)
+    y32 = run_gemm(p, gpu, out_f32=True)
+    assert np.abs(y32 - ref).max() < 2e-4, np.abs(y32 - ref).max()     # fp32 accumulation only
+    y16 = run_gemm(p, gpu)
+    assert np.array_equal(y16.view(np.uint16), y32.astype(np.float16).view(np.uint16))
+    check_layer_output(y16, ref)
+
+
+@pytest.mark.parametrize("k,n", [(4096, 6144), (4096, 28672), (14336, 4096)])
+@pytest.mark.parametrize("m", [1, 8])
+def test_stream_kernel_llama_shapes(gpu, m, k, n):
+    p = make_linear_problem(m, k, n, seed=k + n + m)
+    ref = reference_product(p)
+    y16 = run_gemm(p, gpu)
+    check_layer_output(y16, ref)
+
+
+@pytest.mark.parametrize("m", [17, 33, 64, 65, 130])
+def test_stream_kernel_mid_m(gpu, m):
+    p = make_linear_problem(m, 512, 256, seed=m)
+    ref = reference_product(p, exact=True)
+    y32 = run_gemm(p, gpu, out_f32=True)
+    assert np.abs(y32 - ref).max() < 2e-4
+    check_layer_output(run_gemm(p, gpu), ref)
+
+
+@pytest.mark.parametrize("upw", [1, 2, 4, 8])
+def test_units_per_wave_override(gpu, upw):
+    p = make_linear_problem(2, 1408, 256, seed=upw)     # 11 groups: ragged against 4*upw
+    ref = reference_product(p, exact=True)
+    y32 = run_gemm(p, gpu, out_f32=True, flags=upw << 8)
+    assert np.abs(y32 - ref).max() < 2e-4
+
+
+def test_per_column_scales(gpu):
+    for k in (128, 384):
+        p = make_linear_problem(3, k, 256, seed=k, per_column=True)
+        ref = reference_product(p, exact=True)
+        y32 = run_gemm(p, gpu, out_f32=True)
+        assert np.abs(y32 - ref).max() < 2e-4
+
+
+def test_deterministic_and_repeatable(gpu):
+    p = make_linear_problem(4, 4096, 4096, seed=5)
+    a = run_gemm(p, gpu)
+    b = run_gemm(p, gpu)
+    assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
+
+
+def test_row_stride(gpu):
+    """A may be a row-strided view (lda > k)."""
+    from uniql_amd import ops
+    p = make_linear_problem(4, 256, 256, seed=8)
+    x, b, s = to_gpu(p, gpu)
+    big = torch.zeros(4, 512, dtype=torch.float16, device=gpu)
+    big[:, :256] = x
+    y = ops.w4a16_gemm_ex(big[:, :256], b, s, workspace_for(256, gpu), 4, 256, 256).cpu().numpy()
+    check_layer_output(y, reference_product(p))
+
+
+# ------------------------------------------------------------------ fused rotation
+@pytest.mark.parametrize("m", [1, 5, 16, 40])
+def test_fused_blockwise_hadamard(gpu, m):
+    k, n = 1536, 256           # 12 blocks of 128: not a power of two overall
+    p = make_linear_problem(m, k, n, seed=m + 40)
+    xr = O.fwht(p["x"], 128 ** -0.5, block=128)          # fp16 result of the standalone rotation
+    w = O.dequant_codes(p["q"], p["s"])
+    ref = O.gemm_fp64(xr, w)
+    y32 = run_gemm(p, gpu, out_f32=True, had_block=128, had_scale=128 ** -0.5)
+    assert np.abs(y32 - ref).max() < 2e-4
+    check_layer_output(run_gemm(p, gpu, had_block=128, had_scale=128 ** -0.5), ref)
+
+
+@pytest.mark.parametrize("m", [1, 3])
+def test_full_width_hadamard_prologue(gpu, m):
+    k, n = 8192, 256
+    p = make_linear_problem(m, k, n, seed=m + 80)
+    xr = O.fwht(p["x"], k ** -0.5)
+    ref = O.gemm_fp64(xr, O.dequant_codes(p["q"], p["s"]))
+    y32 = run_gemm(p, gpu, out_f32=True, had_block=k, had_scale=k ** -0.5)
+    assert np.abs(y32 - ref).max() < 2e-4
+
+
+# ------------------------------------------------------------------ error paths
+def test_errors(gpu):
+    from uniql_amd import ops
+    p = make_linear_problem(1, 256, 256)
+    x, b, s = to_gpu(p, gpu)
+    ws = workspace_for(256, gpu)
+    with pytest.raises(RuntimeError):
+        ops.w4a16o16_gemm(x, b, s, ws, 1, 256, 256, True)                 # output_transpose
+    with pytest.raises(RuntimeError):
+        ops.w4a16o16_gemm(x, b, s, ws[:2], 1, 256, 256, False, -1, -1, -1, 16)   # workspace too small
+    with pytest.raises(RuntimeError):
+        ops.w4a16o16_gemm(x.float(), b, s, ws, 1, 256, 256)               # dtype
+    with pytest.raises(RuntimeError):
+        ops.w4a16o16_gemm(x, b, s[:, :128].contiguous(), ws, 1, 256, 256)  # scale shape
+    with pytest.raises(RuntimeError):
+        ops.w4a16o16_gemm(x.cpu(), b, s, ws, 1, 256, 256)                 # no CPU path
+    y = ops.w4a16o16_gemm(x[:0], b, s, ws, 0, 256, 256)
+    assert tuple(y.shape) == (0, 256)

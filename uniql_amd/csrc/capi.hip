@@ -1,0 +1,126 @@
+// extern "C" surface: argument checks and dispatch.  Nothing here allocates,
+// synchronises or throws.
+#include "common.hpp"
+
+namespace uniql {
+int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, int32_t* workspace,
+                  void* scratch, int m, int n, int k, int groups, bool had128, float had_scale, bool out_f32,
+                  int upw_override, hipStream_t stream);
+size_t stream_partial_bytes(int m, int n, int k);
+int dequant_launch(const void* B, const void* S, void* W, uint8_t* codes, int n, int k, int groups,
+                   hipStream_t stream);
+int embedding_launch(const int64_t* ids, int64_t ntokens, const void* weight, const void* scales, void* out,
+                     int64_t vocab, int dim, hipStream_t stream);
+int fwht_launch(const void* x, void* y, int64_t rows, int dim, int block, float scale, int dtype,
+                hipStream_t stream);
+}  // namespace uniql
+
+using namespace uniql;
+
+static inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static inline bool is_pow2(int v) { return v > 0 && (v & (v - 1)) == 0; }
+static inline size_t round256(size_t v) { return (v + 255) & ~(size_t)255; }
+
+static int check_linear_shape(int m, int n, int k, int groups) {
+    if (m < 0 || n <= 0 || k <= 0) return UNIQL_E_SHAPE;
+    if (n % 128 != 0 || k % 128 != 0) return UNIQL_E_SHAPE;
+    if (!(groups == 1 || groups == k / 128)) return UNIQL_E_SHAPE;
+    return UNIQL_OK;
+}
+
+extern "C" {
+
+int uniql_abi_version(void) { return UNIQL_ABI_VERSION; }
+
+const char* uniql_status_string(int code) {
+    switch (code) {
+        case UNIQL_OK: return "ok";
+        case UNIQL_E_NULL: return "a required pointer is NULL";
+        case UNIQL_E_SHAPE: return "sizes violate the packed layout (k % 128, n % 128, groups, dim, block)";
+        case UNIQL_E_ALIGN: return "pointer or leading dimension not 16-byte aligned";
+        case UNIQL_E_WORKSPACE: return "workspace or scratch buffer too small";
+        case UNIQL_E_UNSUPPORTED: return "request not supported by this build";
+        case UNIQL_E_LAUNCH: return "HIP runtime rejected the kernel launch";
+        default: return "unknown status";
+    }
+}
+
+size_t uniql_w4a16_gemm_scratch_bytes(int m, int n, int k, int had_block) {
+    if (m <= 0 || n <= 0 || k <= 0) return 0;
+    size_t bytes = round256(stream_partial_bytes(m, n, k));
+    if (had_block != 0 && had_block != 128) bytes += round256((size_t)m * k * sizeof(half_t));
+    return bytes;
+}
+
+int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, void* D, int32_t* workspace,
+                     int64_t workspace_len, void* scratch, size_t scratch_bytes, int m, int n, int k, int groups,
+                     int had_block, float had_scale, unsigned flags, void* stream) {
+    const int rc = check_linear_shape(m, n, k, groups);
+    if (rc != UNIQL_OK) return rc;
+    if (flags & UNIQL_F_TRANSPOSE_OUT) return UNIQL_E_UNSUPPORTED;
+    if (m == 0) return UNIQL_OK;
+    if (!A || !B || !S || !D || !workspace) return UNIQL_E_NULL;
+    if (lda < k || (lda % 8) != 0) return UNIQL_E_ALIGN;
+    if (!aligned16(A) || !aligned16(B) || !aligned16(S) || !aligned16(D)) return UNIQL_E_ALIGN;
+    if (workspace_len < n / 128) return UNIQL_E_WORKSPACE;
+    if (had_block != 0 && (!is_pow2(had_block) || had_block < 2 || had_block > 32768 || k % had_block != 0))
+        return UNIQL_E_SHAPE;
+    const size_t need = uniql_w4a16_gemm_scratch_bytes(m, n, k, had_block);
+    if (need > 0 && (!scratch || scratch_bytes < need)) return UNIQL_E_WORKSPACE;
+    if (scratch && !aligned16(scratch)) return UNIQL_E_ALIGN;
+    hipStream_t st = reinterpret_cast<hipStream_t>(stream);
+
+    const void* Ain = A;
+    int64_t ld = lda;
+    bool had128 = (had_block == 128);
+    if (had_block != 0 && !had128) {
+        // rotate into the tail of the scratch buffer, then run the plain product on it
+        char* rot = reinterpret_cast<char*>(scratch) + round256(stream_partial_bytes(m, n, k));
+        if (lda != k) {
+            for (int r = 0; r < m; ++r) {
+                const int e = fwht_launch(reinterpret_cast<const half_t*>(A) + (size_t)r * lda,
+                                          reinterpret_cast<half_t*>(rot) + (size_t)r * k, 1, k, had_block, had_scale,
+                                          UNIQL_DT_F16, st);
+                if (e != UNIQL_OK) return e;
+            }
+        } else {
+            const int e = fwht_launch(A, rot, m, k, had_block, had_scale, UNIQL_DT_F16, st);
+            if (e != UNIQL_OK) return e;
+        }
+        Ain = rot;
+        ld = k;
+    }
+    const int upw_override = (int)((flags >> 8) & 0xffu);
+    return stream_launch(Ain, ld, B, S, D, workspace, scratch, m, n, k, groups, had128, had_scale,
+                         (flags & UNIQL_F_OUT_F32) != 0, upw_override, st);
+}
+
+int uniql_w4a16_dequant(const void* B, const void* S, void* W, uint8_t* codes, int n, int k, int groups,
+                        void* stream) {
+    const int rc = check_linear_shape(1, n, k, groups);
+    if (rc != UNIQL_OK) return rc;
+    if (!B || !S || (!W && !codes)) return UNIQL_E_NULL;
+    if (!aligned16(B)) return UNIQL_E_ALIGN;
+    return dequant_launch(B, S, W, codes, n, k, groups, reinterpret_cast<hipStream_t>(stream));
+}
+
+int uniql_w4_embedding_lookup(const int64_t* ids, int64_t ntokens, const void* weight, const void* scales,
+                              void* out, int64_t vocab, int dim, void* stream) {
+    if (ntokens < 0 || vocab <= 0 || dim <= 0 || dim % 8 != 0) return UNIQL_E_SHAPE;
+    if (ntokens == 0) return UNIQL_OK;
+    if (!ids || !weight || !scales || !out) return UNIQL_E_NULL;
+    if (!aligned16(out) || (reinterpret_cast<uintptr_t>(weight) & 3u)) return UNIQL_E_ALIGN;
+    return embedding_launch(ids, ntokens, weight, scales, out, vocab, dim, reinterpret_cast<hipStream_t>(stream));
+}
+
+int uniql_fwht(const void* x, void* y, int64_t rows, int dim, int block, float scale, int dtype, void* stream) {
+    if (dtype != UNIQL_DT_F16 && dtype != UNIQL_DT_BF16 && dtype != UNIQL_DT_F32) return UNIQL_E_UNSUPPORTED;
+    if (rows < 0 || dim <= 0 || !is_pow2(block) || block < 2 || block > 32768 || dim % block != 0)
+        return UNIQL_E_SHAPE;
+    if (rows == 0) return UNIQL_OK;
+    if (!x || !y) return UNIQL_E_NULL;
+    if (block == 128 && dtype == UNIQL_DT_F16 && (!aligned16(x) || !aligned16(y))) return UNIQL_E_ALIGN;
+    return fwht_launch(x, y, rows, dim, block, scale, dtype, reinterpret_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

@@ -1,0 +1,128 @@
+// Walsh-Hadamard transform of fp16 rows: y = fp16((x . H_block) * scale), H the
+// Sylvester (natural-order) matrix, applied to consecutive `block`-wide pieces.
+// Butterflies run in fp32, lowest index bit first, one rounding to fp16 at the end.
+#include "common.hpp"
+
+namespace uniql {
+
+// ---- block == 128: one 16-lane group per piece, all in registers ------------------
+__global__ __launch_bounds__(256) void fwht128_kernel(const u32x4* __restrict__ x, u32x4* __restrict__ y,
+                                                     int64_t pieces, float scale) {
+    const int64_t piece = (int64_t)blockIdx.x * 16 + (threadIdx.x >> 4);
+    const int seg = threadIdx.x & 15;
+    // every lane of a 16-lane group shares `piece`, so the exchange below never
+    // crosses into a group that has left
+    if (piece >= pieces) return;
+    const u32x4 v = x[piece * 16 + seg];
+    float f[8];
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const h2 hv = bits_to_h2(v[p]);
+        f[2 * p] = (float)hv.x;
+        f[2 * p + 1] = (float)hv.y;
+    }
+    wht128_row16(f, seg);
+    u32x4 o;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        h2 hv;
+        hv.x = (half_t)(f[2 * p] * scale);
+        hv.y = (half_t)(f[2 * p + 1] * scale);
+        o[p] = h2_to_bits(hv);
+    }
+    y[piece * 16 + seg] = o;
+}
+
+// ---- general power of two: one workgroup per piece, fp32 image in LDS --------------
+// A pass handles CNT consecutive index bits starting at bit `lo`: each task gathers
+// 2^CNT values whose indices differ only in those bits, runs CNT butterfly stages in
+// registers and scatters them back.
+template <int CNT>
+__device__ __forceinline__ void fwht_pass(float* buf, int L, int lo, int tid, int nthreads) {
+    constexpr int E = 1 << CNT;
+    const int tasks = L >> CNT;
+    const int lowmask = (1 << lo) - 1;
+    for (int t = tid; t < tasks; t += nthreads) {
+        const int base = ((t >> lo) << (lo + CNT)) | (t & lowmask);
+        float v[E];
+#pragma unroll
+        for (int i = 0; i < E; ++i) v[i] = buf[base + (i << lo)];
+#pragma unroll
+        for (int h = 1; h < E; h <<= 1) {
+#pragma unroll
+            for (int i = 0; i < E; ++i) {
+                if ((i & h) == 0) {
+                    const float p = v[i], q = v[i + h];
+                    v[i] = p + q;
+                    v[i + h] = p - q;
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < E; ++i) buf[base + (i << lo)] = v[i];
+    }
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void fwht_lds_kernel(const T* __restrict__ x, T* __restrict__ y, int L,
+                                                      int log2L, float scale) {
+    extern __shared__ __attribute__((aligned(16))) float fbuf[];
+    const int tid = threadIdx.x;
+    const T* xp = x + (size_t)blockIdx.x * L;
+    T* yp = y + (size_t)blockIdx.x * L;
+    for (int i = tid; i < L; i += 256) fbuf[i] = (float)xp[i];
+    __syncthreads();
+    int lo = 0;
+    while (lo < log2L) {
+        const int left = log2L - lo;
+        if (left >= 3) {
+            fwht_pass<3>(fbuf, L, lo, tid, 256);
+            lo += 3;
+        } else if (left == 2) {
+            fwht_pass<2>(fbuf, L, lo, tid, 256);
+            lo += 2;
+        } else {
+            fwht_pass<1>(fbuf, L, lo, tid, 256);
+            lo += 1;
+        }
+        __syncthreads();
+    }
+    for (int i = tid; i < L; i += 256) yp[i] = (T)(fbuf[i] * scale);
+}
+
+template <typename T>
+static int fwht_lds_launch(const void* x, void* y, int64_t pieces, int block, float scale, hipStream_t stream) {
+    int log2L = 0;
+    while ((1 << log2L) < block) ++log2L;
+    const size_t shmem = (size_t)block * sizeof(float);
+    if (shmem > 64 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&fwht_lds_kernel<T>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
+            return UNIQL_E_LAUNCH;
+    }
+    hipLaunchKernelGGL((fwht_lds_kernel<T>), dim3((unsigned)pieces), dim3(256), shmem, stream,
+                       reinterpret_cast<const T*>(x), reinterpret_cast<T*>(y), block, log2L, scale);
+    return UNIQL_OK;
+}
+
+int fwht_launch(const void* x, void* y, int64_t rows, int dim, int block, float scale, int dtype,
+                hipStream_t stream) {
+    const int64_t pieces = rows * (dim / block);
+    if (pieces == 0) return UNIQL_OK;
+    if (block == 128 && dtype == UNIQL_DT_F16) {
+        const int64_t grid = (pieces + 15) / 16;
+        if (grid > 0x7fffffffLL) return UNIQL_E_SHAPE;
+        hipLaunchKernelGGL(fwht128_kernel, dim3((unsigned)grid), dim3(256), 0, stream,
+                           reinterpret_cast<const u32x4*>(x), reinterpret_cast<u32x4*>(y), pieces, scale);
+    } else {
+        if (pieces > 0x7fffffffLL) return UNIQL_E_SHAPE;
+        int rc;
+        if (dtype == UNIQL_DT_F16) rc = fwht_lds_launch<half_t>(x, y, pieces, block, scale, stream);
+        else if (dtype == UNIQL_DT_BF16) rc = fwht_lds_launch<__bf16>(x, y, pieces, block, scale, stream);
+        else rc = fwht_lds_launch<float>(x, y, pieces, block, scale, stream);
+        if (rc != UNIQL_OK) return rc;
+    }
+    return hipGetLastError() == hipSuccess ? UNIQL_OK : UNIQL_E_LAUNCH;
+}
+
+}  // namespace uniql

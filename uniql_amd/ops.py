@@ -1,0 +1,177 @@
+"""Extension-level operators: the functions the reference's compiled modules
+export, with the same positional arguments, backed by the C ABI.
+
+    w4a16o16_gemm           <- quant_linear_cuda          (csrc/linear/quant_linear.cpp:6-24)
+    w4a16_embedding_lookup  <- quant_embedding_cuda       (csrc/embedding/quant_embedding.cpp:3-8)
+    fast_hadamard_transform <- fast_hadamard_transform_cuda (quantize/hadamard_helpers.py:22-35)
+
+Outputs are allocated with torch.empty on the input's device and kernels are
+enqueued on torch's current stream, so calls are valid inside
+torch.cuda.graph capture.  Errors surface as RuntimeError.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _capi
+
+__all__ = [
+    "w4a16o16_gemm", "w4a16_gemm_ex", "w4a16_dequant", "w4a16_embedding_lookup",
+    "fast_hadamard_transform", "hadamard_blockwise", "unsupported_hadamard_variant",
+]
+
+
+def _stream_ptr(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def _require_gpu(t: torch.Tensor, name: str) -> None:
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a GPU tensor (this package has no CPU path)")
+
+
+def w4a16_gemm_ex(A: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: torch.Tensor,
+                  size_m: int, size_n: int, size_k: int, *, had_block: int = 0,
+                  had_scale: float = 1.0, out_f32: bool = False, flags: int = 0) -> torch.Tensor:
+    """D[m, n] = rotate(A)[m, k] . dequant(B)[k, n].  `had_block` 0 means no rotation."""
+    for t, name in ((A, "A"), (B, "B"), (s, "s"), (workspace, "workspace")):
+        _require_gpu(t, name)
+    if A.dtype != torch.float16 or s.dtype != torch.float16:
+        raise RuntimeError("A and s must be float16")
+    if B.dtype != torch.int32 or workspace.dtype != torch.int32:
+        raise RuntimeError("B and workspace must be int32")
+    if A.dim() != 2 or A.stride(1) != 1:
+        raise RuntimeError("A must be 2-D with unit stride along K")
+    if A.shape[0] != size_m or A.shape[1] != size_k:
+        raise RuntimeError(f"A is {tuple(A.shape)}, expected ({size_m}, {size_k})")
+    if not (B.is_contiguous() and s.is_contiguous() and workspace.is_contiguous()):
+        raise RuntimeError("B, s and workspace must be contiguous")
+    if tuple(B.shape) != (size_k // 16, 2 * size_n):
+        raise RuntimeError(f"B is {tuple(B.shape)}, expected ({size_k // 16}, {2 * size_n})")
+    if s.dim() != 2 or s.shape[1] != size_n:
+        raise RuntimeError(f"s is {tuple(s.shape)}, expected (groups, {size_n})")
+    groups = s.shape[0]
+    # same test as the reference wrapper (marlin_gemm_kernel.cuh:1008-1010)
+    if groups != 1 and (size_k // groups) * groups != size_k:
+        raise RuntimeError(f"k={size_k} not compatible with {groups} groups.")
+    lib = _capi.load()
+    dev = A.device
+    out_dtype = torch.float32 if out_f32 else torch.float16
+    with torch.cuda.device(dev):
+        D = torch.empty((size_m, size_n), dtype=out_dtype, device=dev)
+        need = lib.uniql_w4a16_gemm_scratch_bytes(size_m, size_n, size_k, had_block)
+        scratch = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
+        if out_f32:
+            flags |= _capi.F_OUT_F32
+        lda = A.stride(0) if size_m > 1 else size_k
+        code = lib.uniql_w4a16_gemm(
+            A.data_ptr(), lda, B.data_ptr(), s.data_ptr(), D.data_ptr(),
+            workspace.data_ptr(), workspace.numel(),
+            scratch.data_ptr() if scratch is not None else None, need,
+            size_m, size_n, size_k, groups, had_block, float(had_scale), flags, _stream_ptr(dev))
+    _capi.check(code, "uniql_w4a16_gemm")
+    return D
+
+
+def w4a16o16_gemm(A, B, s, workspace, size_m, size_n, size_k, output_transpose=False,
+                  thread_k=-1, thread_n=-1, sms=-1, max_par=8):
+    """Same call as the reference extension.  thread_k / thread_n / sms choose
+    CUDA tile shapes there and are accepted and ignored; max_par only sizes the
+    reference's lock array, the same check is applied to `workspace`."""
+    if output_transpose:
+        raise RuntimeError("output_transpose=True is not supported (the reference's Python never passes it)")
+    if workspace.numel() < size_n // 128 * max_par:
+        raise RuntimeError(f"workspace must be of size at least {size_n // 128 * max_par}.")
+    return w4a16_gemm_ex(A, B, s, workspace, int(size_m), int(size_n), int(size_k))
+
+
+def w4a16_dequant(B: torch.Tensor, s: torch.Tensor, size_n: int, size_k: int, want_codes: bool = False):
+    """Natural-order dequantised weights fp16 [k, n] (and the raw codes uint8 [k, n])."""
+    _require_gpu(B, "B")
+    _require_gpu(s, "s")
+    if B.dtype != torch.int32 or s.dtype != torch.float16 or not (B.is_contiguous() and s.is_contiguous()):
+        raise RuntimeError("B must be contiguous int32 and s contiguous float16")
+    if tuple(B.shape) != (size_k // 16, 2 * size_n) or s.dim() != 2 or s.shape[1] != size_n:
+        raise RuntimeError("B / s shapes do not match size_k, size_n")
+    lib = _capi.load()
+    dev = B.device
+    with torch.cuda.device(dev):
+        W = torch.empty((size_k, size_n), dtype=torch.float16, device=dev)
+        codes = torch.empty((size_k, size_n), dtype=torch.uint8, device=dev) if want_codes else None
+        code = lib.uniql_w4a16_dequant(B.data_ptr(), s.data_ptr(), W.data_ptr(),
+                                       codes.data_ptr() if want_codes else None,
+                                       size_n, size_k, s.shape[0], _stream_ptr(dev))
+    _capi.check(code, "uniql_w4a16_dequant")
+    return (W, codes) if want_codes else W
+
+
+def w4a16_embedding_lookup(input: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
+    """out[..., :] = (code - 8) * scale[id].  Checks follow quant_embedding_kernel.cuh:121-134."""
+    if weight.dim() != 2:
+        raise RuntimeError("weight must be 2-D")
+    _require_gpu(weight, "weight")
+    if weight.dtype != torch.int32:
+        raise RuntimeError("weight's dtype must be int32")
+    vocab, words = weight.shape
+    dim = words * 8
+    if scale.dim() != 1:
+        raise RuntimeError("scale must be 1-D")
+    _require_gpu(scale, "scale")
+    if scale.dtype != torch.float16:
+        raise RuntimeError("scale's dtype must be float16")
+    if scale.numel() != vocab:
+        raise RuntimeError("scale must have one entry per vocabulary row")
+    if input.dim() not in (1, 2):
+        raise RuntimeError("input must be a 1D or 2D tensor")
+    _require_gpu(input, "input")
+    if input.dtype != torch.int64:
+        raise RuntimeError("input's dtype must be int64")
+    lib = _capi.load()
+    dev = input.device
+    ids = input.contiguous()
+    weight_c = weight.detach()
+    if not weight_c.is_contiguous() or not scale.is_contiguous():
+        raise RuntimeError("weight and scale must be contiguous")
+    with torch.cuda.device(dev):
+        out = torch.empty((*ids.shape, dim), dtype=torch.float16, device=dev)
+        code = lib.uniql_w4_embedding_lookup(ids.data_ptr(), ids.numel(), weight_c.data_ptr(), scale.data_ptr(),
+                                             out.data_ptr(), vocab, dim, _stream_ptr(dev))
+    _capi.check(code, "uniql_w4_embedding_lookup")
+    return out
+
+
+def hadamard_blockwise(x: torch.Tensor, scale: float, block: int | None = None) -> torch.Tensor:
+    """(x . H_block) * scale on consecutive block-wide pieces of the last axis; new tensor."""
+    _require_gpu(x, "x")
+    dim = x.shape[-1]
+    block = dim if block is None else block
+    dtypes = {torch.float16: _capi.DT_F16, torch.bfloat16: _capi.DT_BF16, torch.float32: _capi.DT_F32}
+    if x.dtype not in dtypes:
+        raise RuntimeError(f"hadamard transform supports float16 / bfloat16 / float32, got {x.dtype}")
+    lib = _capi.load()
+    xc = x.contiguous()
+    dev = x.device
+    with torch.cuda.device(dev):
+        y = torch.empty_like(xc)
+        rows = xc.numel() // dim if dim else 0
+        code = lib.uniql_fwht(xc.data_ptr(), y.data_ptr(), rows, dim, block, float(scale),
+                              dtypes[x.dtype], _stream_ptr(dev))
+    _capi.check(code, "uniql_fwht")
+    return y
+
+
+def fast_hadamard_transform(x: torch.Tensor, scale: float = 1.0) -> torch.Tensor:
+    """Power-of-two Walsh-Hadamard transform along the last axis, times scale."""
+    dim = x.shape[-1]
+    if dim & (dim - 1):
+        raise RuntimeError(f"fast_hadamard_transform needs a power-of-two width, got {dim}")
+    return hadamard_blockwise(x, scale, dim)
+
+
+def unsupported_hadamard_variant(base: int):
+    def _fn(x, scale=1.0):
+        raise NotImplementedError(
+            f"fast_hadamard_transform_{base}N: the {base}x{base} base matrix comes from a third-party "
+            "package that is not part of the reference tree; only power-of-two widths are implemented")
+    _fn.__name__ = f"fast_hadamard_transform_{base}N"
+    return _fn
