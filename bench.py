@@ -82,8 +82,10 @@ class Layer:
 
 
 def time_graphs(run_step, n_variants, steps, warmup):
-    """Captures run_step(i) for i < n_variants as HIP graphs, replays them round-robin and
-    returns seconds per step measured with events on the launch stream."""
+    """Times exactly `steps` calls of run_step(i), i cycling over n_variants, as HIP graph
+    replays: one graph holds n_variants consecutive steps (a second, shorter one the
+    remainder), so the per-replay launch cost is shared by many kernels.  Returns
+    (seconds per step from events on the launch stream, wall seconds per step)."""
     import torch
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -92,20 +94,27 @@ def time_graphs(run_step, n_variants, steps, warmup):
             run_step(i)
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
-    graphs, keep = [], []
-    for i in range(n_variants):
+    keep = []
+
+    def capture(count):
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
-            keep.append(run_step(i))
-        graphs.append(g)
-    for i in range(warmup):
-        graphs[i % n_variants].replay()
+            for i in range(count):
+                keep.append(run_step(i))
+        return g
+
+    full = capture(n_variants)
+    rest = capture(steps % n_variants) if steps % n_variants else None
+    for _ in range(max(1, warmup // n_variants)):
+        full.replay()
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     start.record()
-    for i in range(steps):
-        graphs[i % n_variants].replay()
+    for _ in range(steps // n_variants):
+        full.replay()
+    if rest is not None:
+        rest.replay()
     stop.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0

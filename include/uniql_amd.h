@@ -27,7 +27,7 @@ enum {
     UNIQL_E_NULL = -1,        /* a required pointer is NULL                        */
     UNIQL_E_SHAPE = -2,       /* m/n/k/groups violate the layout's divisibility    */
     UNIQL_E_ALIGN = -3,       /* a pointer or leading dimension is not 16-byte aligned */
-    UNIQL_E_WORKSPACE = -4,   /* workspace or scratch too small                    */
+    UNIQL_E_WORKSPACE = -4,   /* workspace, accum or temp buffer too small         */
     UNIQL_E_UNSUPPORTED = -5, /* valid request this build does not implement       */
     UNIQL_E_LAUNCH = -6       /* the HIP runtime rejected a launch                 */
 };
@@ -38,7 +38,8 @@ enum {
     UNIQL_F_FORCE_SKINNY = 1 << 1, /* use the weight-streaming kernel whatever m is */
     UNIQL_F_FORCE_TILED = 1 << 2,  /* use the prefill (LDS + MFMA tile) kernel whatever m is */
     UNIQL_F_TRANSPOSE_OUT = 1 << 3 /* reference's output_transpose; rejected with UNIQL_E_UNSUPPORTED */
-    /* bits 8..15: units-per-wave override for the skinny kernel (0 = heuristic); tuning hook */
+    /* tuning hooks of the streaming kernel, 0 = choose: bits 8..15 K-groups per wavefront,
+       bits 16..19 wavefronts per workgroup (4, 8 or 16), bit 20 disables the register prefetch */
 };
 
 int uniql_abi_version(void);
@@ -55,24 +56,37 @@ const char* uniql_status_string(int code);
  *   S          device, fp16 [groups, n], permuted by quantize_helpers.py:168-180;
  *              groups == k/128 (group-128 scales) or groups == 1 (one scale per column)
  *   D          device, fp16 [m, n] row-major (float32 with UNIQL_F_OUT_F32)
- *   workspace  device, int32 [workspace_len] >= n/128 entries, all zero on entry;
- *              zero again when the kernels have finished (the module's
- *              `workspace` buffer, quantize/quant_linear_layers.py:33-35)
- *   scratch    device, at least uniql_w4a16_gemm_scratch_bytes(m, n, k) bytes,
- *              contents irrelevant (replaces the reference's per-call `C`
- *              allocation, marlin_gemm_kernel.cuh:1018); may be NULL if that size is 0
+ *   workspace  device, int32 [workspace_len] or NULL: the module's `workspace` buffer
+ *              (quantize/quant_linear_layers.py:33-35; the reference's inter-block
+ *              lock array).  Only its length is checked (>= n/128, as the reference
+ *              checks it); it is never read or written, so it stays zero.
+ *   accum      device, uniql_w4a16_gemm_accum_bytes(m, n, k) bytes, ALL ZERO on entry
+ *              and all zero again when the kernels have finished: 64-bit sum|count
+ *              words through which workgroups that share an output column combine
+ *              their partial sums (replaces the reference's per-call fp16 `C`
+ *              buffer and its locks, marlin_gemm_kernel.cuh:515-570,1018).  A caller
+ *              clears it once and reuses it for every call on the same stream; two
+ *              calls that may run concurrently need separate buffers.  May be NULL
+ *              when the size is 0.
+ *   temp       device, uniql_w4a16_gemm_temp_bytes(m, n, k, had_block) bytes, contents
+ *              irrelevant (rotated activations when had_block is neither 0 nor 128);
+ *              may be NULL when that size is 0
  *   had_block  0: none.  Otherwise the activations are rotated first,
  *              A <- fp16(A . H_had_block * had_scale) on consecutive
  *              had_block-wide pieces of each row: 128 is fused into the
  *              streaming kernel's prologue, any other power of two (<= 32768,
- *              dividing k) runs the transform kernel into scratch first.
+ *              dividing k) runs the transform kernel into `temp` first.
  *   k % 128 == 0, n % 128 == 0 (the module pads n to 256).
+ *
+ * Partial sums that meet in `accum` are rounded to multiples of 2^-24 and clamped to
+ * +-2^22 (far beyond the fp16 range of D); NaN partials are not propagated through it.
  */
-size_t uniql_w4a16_gemm_scratch_bytes(int m, int n, int k, int had_block);
+size_t uniql_w4a16_gemm_accum_bytes(int m, int n, int k);
+size_t uniql_w4a16_gemm_temp_bytes(int m, int n, int k, int had_block);
 
 int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, void* D,
-                     int32_t* workspace, int64_t workspace_len,
-                     void* scratch, size_t scratch_bytes,
+                     const int32_t* workspace, int64_t workspace_len,
+                     void* accum, size_t accum_bytes, void* temp, size_t temp_bytes,
                      int m, int n, int k, int groups,
                      int had_block, float had_scale,
                      unsigned flags, void* stream);

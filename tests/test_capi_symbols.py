@@ -39,22 +39,24 @@ def test_host_only_entry_points(lib):
     assert lib.uniql_abi_version() == 1
     assert lib.uniql_status_string(0) == b"ok"
     assert b"NULL" in lib.uniql_status_string(-1)
-    # split-K partials: ceil(K/128/4) * m * n floats, rounded up to 256 bytes
-    assert lib.uniql_w4a16_gemm_scratch_bytes(1, 4096, 4096, 0) == 8 * 1 * 4096 * 4
-    assert lib.uniql_w4a16_gemm_scratch_bytes(1, 4096, 512, 0) == 0
-    extra = lib.uniql_w4a16_gemm_scratch_bytes(2, 4096, 8192, 8192) - lib.uniql_w4a16_gemm_scratch_bytes(2, 4096, 8192, 0)
-    assert extra == 2 * 8192 * 2
+    # one 64-bit word per output element of a (<= 64 row) slab when K can be split
+    assert lib.uniql_w4a16_gemm_accum_bytes(1, 4096, 4096) == 4096 * 8
+    assert lib.uniql_w4a16_gemm_accum_bytes(100, 4096, 4096) == 64 * 4096 * 8
+    assert lib.uniql_w4a16_gemm_accum_bytes(1, 4096, 512) == 0
+    assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 8192) == 2 * 8192 * 2
+    assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 128) == 0
+    assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 0) == 0
 
 
 def test_argument_checks_need_no_gpu(lib):
     """Shape errors are reported before anything touches the device."""
     f = lib.uniql_w4a16_gemm
-    assert f(None, 4096, None, None, None, None, 0, None, 0, 1, 4096 + 64, 4096, 32, 0, 1.0, 0, None) == -2
-    assert f(None, 4096, None, None, None, None, 0, None, 0, 1, 4096, 4096 + 16, 32, 0, 1.0, 0, None) == -2
-    assert f(None, 4096, None, None, None, None, 0, None, 0, 1, 4096, 4096, 7, 0, 1.0, 0, None) == -2
-    assert f(None, 4096, None, None, None, None, 0, None, 0, 1, 4096, 4096, 32, 0, 1.0, 8, None) == -5
-    assert f(None, 4096, None, None, None, None, 0, None, 0, 1, 4096, 4096, 32, 0, 1.0, 0, None) == -1
-    assert f(None, 4096, None, None, None, None, 0, None, 0, 0, 4096, 4096, 32, 0, 1.0, 0, None) == 0
+    assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 1, 4096 + 64, 4096, 32, 0, 1.0, 0, None) == -2
+    assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 1, 4096, 4096 + 16, 32, 0, 1.0, 0, None) == -2
+    assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 1, 4096, 4096, 7, 0, 1.0, 0, None) == -2
+    assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 1, 4096, 4096, 32, 0, 1.0, 8, None) == -5
+    assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 1, 4096, 4096, 32, 0, 1.0, 0, None) == -1
+    assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 0, 4096, 4096, 32, 0, 1.0, 0, None) == 0
     assert lib.uniql_fwht(None, None, 4, 96, 96, 1.0, 0, None) == -2
     assert lib.uniql_fwht(None, None, 4, 128, 128, 1.0, 7, None) == -5
     assert lib.uniql_w4_embedding_lookup(None, 5, None, None, None, 10, 12, None) == -2

@@ -22,9 +22,10 @@ DT_F16, DT_BF16, DT_F32 = 0, 1, 2
 SIGNATURES = {
     "uniql_abi_version": (c_int, []),
     "uniql_status_string": (c_char_p, [c_int]),
-    "uniql_w4a16_gemm_scratch_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
+    "uniql_w4a16_gemm_accum_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "uniql_w4a16_gemm_temp_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "uniql_w4a16_gemm": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
-                                 c_void_p, c_int64, c_void_p, c_size_t,
+                                 c_void_p, c_int64, c_void_p, c_size_t, c_void_p, c_size_t,
                                  c_int, c_int, c_int, c_int, c_int, c_float, c_uint, c_void_p]),
     "uniql_w4a16_dequant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "uniql_w4_embedding_lookup": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p,

@@ -3,10 +3,10 @@
 #include "common.hpp"
 
 namespace uniql {
-int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, int32_t* workspace,
-                  void* scratch, int m, int n, int k, int groups, bool had128, float had_scale, bool out_f32,
-                  int upw_override, hipStream_t stream);
-size_t stream_partial_bytes(int m, int n, int k);
+int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, void* accum, int m, int n,
+                  int k, int groups, bool had128, float had_scale, bool out_f32, unsigned tune,
+                  hipStream_t stream);
+size_t stream_accum_bytes(int m, int n, int k);
 int dequant_launch(const void* B, const void* S, void* W, uint8_t* codes, int n, int k, int groups,
                    hipStream_t stream);
 int embedding_launch(const int64_t* ids, int64_t ntokens, const void* weight, const void* scales, void* out,
@@ -38,61 +38,66 @@ const char* uniql_status_string(int code) {
         case UNIQL_E_NULL: return "a required pointer is NULL";
         case UNIQL_E_SHAPE: return "sizes violate the packed layout (k % 128, n % 128, groups, dim, block)";
         case UNIQL_E_ALIGN: return "pointer or leading dimension not 16-byte aligned";
-        case UNIQL_E_WORKSPACE: return "workspace or scratch buffer too small";
+        case UNIQL_E_WORKSPACE: return "workspace, accum or temp buffer too small";
         case UNIQL_E_UNSUPPORTED: return "request not supported by this build";
         case UNIQL_E_LAUNCH: return "HIP runtime rejected the kernel launch";
         default: return "unknown status";
     }
 }
 
-size_t uniql_w4a16_gemm_scratch_bytes(int m, int n, int k, int had_block) {
+size_t uniql_w4a16_gemm_accum_bytes(int m, int n, int k) {
     if (m <= 0 || n <= 0 || k <= 0) return 0;
-    size_t bytes = round256(stream_partial_bytes(m, n, k));
-    if (had_block != 0 && had_block != 128) bytes += round256((size_t)m * k * sizeof(half_t));
-    return bytes;
+    return round256(stream_accum_bytes(m, n, k));
 }
 
-int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, void* D, int32_t* workspace,
-                     int64_t workspace_len, void* scratch, size_t scratch_bytes, int m, int n, int k, int groups,
-                     int had_block, float had_scale, unsigned flags, void* stream) {
+size_t uniql_w4a16_gemm_temp_bytes(int m, int n, int k, int had_block) {
+    if (m <= 0 || n <= 0 || k <= 0) return 0;
+    if (had_block != 0 && had_block != 128) return round256((size_t)m * k * sizeof(half_t));
+    return 0;
+}
+
+int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, void* D, const int32_t* workspace,
+                     int64_t workspace_len, void* accum, size_t accum_bytes, void* temp, size_t temp_bytes, int m,
+                     int n, int k, int groups, int had_block, float had_scale, unsigned flags, void* stream) {
     const int rc = check_linear_shape(m, n, k, groups);
     if (rc != UNIQL_OK) return rc;
     if (flags & UNIQL_F_TRANSPOSE_OUT) return UNIQL_E_UNSUPPORTED;
     if (m == 0) return UNIQL_OK;
-    if (!A || !B || !S || !D || !workspace) return UNIQL_E_NULL;
+    if (!A || !B || !S || !D) return UNIQL_E_NULL;
     if (lda < k || (lda % 8) != 0) return UNIQL_E_ALIGN;
     if (!aligned16(A) || !aligned16(B) || !aligned16(S) || !aligned16(D)) return UNIQL_E_ALIGN;
-    if (workspace_len < n / 128) return UNIQL_E_WORKSPACE;
+    if (workspace && workspace_len < n / 128) return UNIQL_E_WORKSPACE;
     if (had_block != 0 && (!is_pow2(had_block) || had_block < 2 || had_block > 32768 || k % had_block != 0))
         return UNIQL_E_SHAPE;
-    const size_t need = uniql_w4a16_gemm_scratch_bytes(m, n, k, had_block);
-    if (need > 0 && (!scratch || scratch_bytes < need)) return UNIQL_E_WORKSPACE;
-    if (scratch && !aligned16(scratch)) return UNIQL_E_ALIGN;
+    const size_t need_accum = uniql_w4a16_gemm_accum_bytes(m, n, k);
+    if (need_accum > 0 && (!accum || accum_bytes < need_accum)) return UNIQL_E_WORKSPACE;
+    const size_t need_temp = uniql_w4a16_gemm_temp_bytes(m, n, k, had_block);
+    if (need_temp > 0 && (!temp || temp_bytes < need_temp)) return UNIQL_E_WORKSPACE;
+    if ((accum && !aligned16(accum)) || (temp && !aligned16(temp))) return UNIQL_E_ALIGN;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 
     const void* Ain = A;
     int64_t ld = lda;
-    bool had128 = (had_block == 128);
+    const bool had128 = (had_block == 128);
     if (had_block != 0 && !had128) {
-        // rotate into the tail of the scratch buffer, then run the plain product on it
-        char* rot = reinterpret_cast<char*>(scratch) + round256(stream_partial_bytes(m, n, k));
+        // rotate into the temporary buffer, then run the plain product on it
         if (lda != k) {
             for (int r = 0; r < m; ++r) {
                 const int e = fwht_launch(reinterpret_cast<const half_t*>(A) + (size_t)r * lda,
-                                          reinterpret_cast<half_t*>(rot) + (size_t)r * k, 1, k, had_block, had_scale,
+                                          reinterpret_cast<half_t*>(temp) + (size_t)r * k, 1, k, had_block, had_scale,
                                           UNIQL_DT_F16, st);
                 if (e != UNIQL_OK) return e;
             }
         } else {
-            const int e = fwht_launch(A, rot, m, k, had_block, had_scale, UNIQL_DT_F16, st);
+            const int e = fwht_launch(A, temp, m, k, had_block, had_scale, UNIQL_DT_F16, st);
             if (e != UNIQL_OK) return e;
         }
-        Ain = rot;
+        Ain = temp;
         ld = k;
     }
-    const int upw_override = (int)((flags >> 8) & 0xffu);
-    return stream_launch(Ain, ld, B, S, D, workspace, scratch, m, n, k, groups, had128, had_scale,
-                         (flags & UNIQL_F_OUT_F32) != 0, upw_override, st);
+    const unsigned tune = flags >> 8;  // tuning fields, see the header
+    return stream_launch(Ain, ld, B, S, D, accum, m, n, k, groups, had128, had_scale,
+                         (flags & UNIQL_F_OUT_F32) != 0, tune, st);
 }
 
 int uniql_w4a16_dequant(const void* B, const void* S, void* W, uint8_t* codes, int n, int k, int groups,

@@ -29,12 +29,43 @@ __device__ __forceinline__ uint32_t h2_to_bits(h2 v) { return __builtin_bit_cast
 //              makes the fp16 number 1024 + code; subtracting 1032 leaves code - 8.
 //   high form: codes sit in bits 4..7 and 20..23, giving 1024 + 16*code;
 //              (1024 + 16 c) / 16 - 72 = c - 8.  Every step is exact in fp16.
+// The masks and the exponent pattern are kept in registers (not literals): gfx950's
+// three-operand v_and_or_b32 cannot encode literals, and with literals the compiler
+// falls back to a separate AND and OR.
+struct NibbleMagic {
+    uint32_t mask_low, mask_high, exponent;
+    __device__ __forceinline__ void init() {
+        mask_low = 0x000f000fu;
+        mask_high = 0x00f000f0u;
+        exponent = 0x64006400u;
+        asm volatile("" : "+v"(mask_low), "+v"(mask_high));
+        asm volatile("" : "+s"(exponent));
+    }
+    __device__ __forceinline__ h2 pair_low(uint32_t q) const {
+        return bits_to_h2((q & mask_low) | exponent) - h2{(half_t)1032.0f, (half_t)1032.0f};
+    }
+    __device__ __forceinline__ h2 pair_high(uint32_t q) const {
+        return bits_to_h2((q & mask_high) | exponent) * h2{(half_t)0.0625f, (half_t)0.0625f} -
+               h2{(half_t)72.0f, (half_t)72.0f};
+    }
+};
 __device__ __forceinline__ h2 code_pair_low(uint32_t q) {
     return bits_to_h2((q & 0x000f000fu) | 0x64006400u) - h2{(half_t)1032.0f, (half_t)1032.0f};
 }
 __device__ __forceinline__ h2 code_pair_high(uint32_t q) {
     return bits_to_h2((q & 0x00f000f0u) | 0x64006400u) * h2{(half_t)0.0625f, (half_t)0.0625f}
            - h2{(half_t)72.0f, (half_t)72.0f};
+}
+
+// fp16(v * s) with two roundings (fp32 product, then fp16), the result a separate
+// multiply and conversion give.  Written as one expression the compiler selects
+// v_fma_mixlo_f16, which rounds the exact product once and differs in rare cases; the
+// empty asm keeps the product a plain fp32 value so that every kernel (and the
+// fp32 host model of the transform) rounds the same way.
+__device__ __forceinline__ half_t scaled_to_half(float v, float s) {
+    float p = v * s;
+    asm volatile("" : "+v"(p));
+    return (half_t)p;
 }
 
 // Where each lane's eight scale values sit for a 16-byte load, grouped case:

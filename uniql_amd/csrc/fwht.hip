@@ -26,8 +26,8 @@ __global__ __launch_bounds__(256) void fwht128_kernel(const u32x4* __restrict__ 
 #pragma unroll
     for (int p = 0; p < 4; ++p) {
         h2 hv;
-        hv.x = (half_t)(f[2 * p] * scale);
-        hv.y = (half_t)(f[2 * p + 1] * scale);
+        hv.x = scaled_to_half(f[2 * p], scale);
+        hv.y = scaled_to_half(f[2 * p + 1], scale);
         o[p] = h2_to_bits(hv);
     }
     y[piece * 16 + seg] = o;
@@ -87,7 +87,11 @@ __global__ __launch_bounds__(256) void fwht_lds_kernel(const T* __restrict__ x, 
         }
         __syncthreads();
     }
-    for (int i = tid; i < L; i += 256) yp[i] = (T)(fbuf[i] * scale);
+    for (int i = tid; i < L; i += 256) {
+        float p = fbuf[i] * scale;
+        asm volatile("" : "+v"(p));  // see scaled_to_half: keep multiply and rounding separate
+        yp[i] = (T)p;
+    }
 }
 
 template <typename T>

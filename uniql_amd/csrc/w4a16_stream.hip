@@ -18,14 +18,19 @@
 //
 // Work split: unit = (strip of 128 columns) x (group of 128 K).  A wave owns `upw`
 // consecutive groups of a strip, the four waves of a workgroup own consecutive
-// group ranges, partial sums meet in LDS.  When K is split over several workgroups
-// they store fp32 partials; the last workgroup to arrive (a counter in `workspace`,
-// which it resets to zero) adds them in a fixed order, so results are
-// deterministic and no workgroup ever waits for another.
+// group ranges, partial sums meet in LDS.  When K is split over several workgroups,
+// each output element has a 64-bit word in a zero-initialised accumulator: bits 8..63
+// hold the running sum as a fixed-point integer (2^-24 units), bits 0..7 the number of
+// contributions.  A workgroup adds (value << 8) + 1 with ONE device-scope atomic and
+// looks at the returned old word: whoever sees count == splits - 1 was last, owns the
+// total (old + own), stores the output and writes the word back to zero.  Integer adds
+// commute, so the result does not depend on arrival order, and nobody waits for anyone.
 #include "common.hpp"
 
 namespace uniql {
 
+constexpr float kAccumScale = 16777216.0f;  // 2^24 fixed-point units per 1.0
+constexpr float kAccumClamp = 4194304.0f;   // 2^22
 constexpr int kXsStride = 68;  // dwords per staged activation row: 64 + 4, keeps the 64 lanes on distinct banks
 
 struct StreamArgs {
@@ -33,28 +38,37 @@ struct StreamArgs {
     const half_t* S;      // permuted scales [groups][N]
     const half_t* X;      // activations [M][ldx]
     void* D;              // fp16 or fp32 [M][N]
-    float* partial;       // [splits][M][N] when splits > 1
-    int32_t* counters;    // [N/128], zero on entry and on exit
+    unsigned long long* accum;  // [M][N] fixed-point sum | count words, zero on entry and on exit (splits > 1)
     int64_t ldx;
     int M, N, K;
     int G;                // number of 128-wide K groups = K/128
     int per_column;       // 1: a single scale row (per-column scales)
     int upw;              // groups per wave
     int splits;           // workgroups along K per strip
+    int xrows;            // activation rows staged per wave: multiple of 4, >= min(M, 16 MT)
     int out_f32;
     float had_scale;
 };
 
-// Registers: MT = 1 needs ~140 VGPRs, which allows 3 waves per SIMD (12 per CU, 96 KiB
-// of weight loads in flight per CU); the bigger M tiles trade occupancy for accumulators.
-template <int MT, bool HAD>
-__global__ __launch_bounds__(256, (MT == 1 ? 3 : (MT == 2 ? 2 : 1))) void w4a16_stream_kernel(const StreamArgs a) {
+__device__ __forceinline__ void store_out(const StreamArgs& a, int m, int n, float v) {
+    if (a.out_f32)
+        reinterpret_cast<float*>(a.D)[(size_t)m * a.N + n] = v;
+    else
+        reinterpret_cast<half_t*>(a.D)[(size_t)m * a.N + n] = (half_t)v;
+}
+
+// MT: 16-row tiles of M per workgroup.  WAVES: wavefronts per workgroup (4, 8 or 16);
+// with 16 a workgroup can cover all of K for shapes with many strips, which removes the
+// exchange of partial sums between workgroups.  PF: prefetch the next group's weights
+// into a second register set while the current one is consumed.
+template <int MT, bool HAD, int WAVES, bool PF>
+__global__ __launch_bounds__(64 * WAVES, (MT == 1 ? (WAVES == 16 ? 4 : 3) : (MT == 2 ? 2 : 1)))
+void w4a16_stream_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
-    __shared__ int s_last;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int w = tid >> 6;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: keeps address math scalar
     const int slot = lane & 15;
     const int kq = lane >> 4;
     const int c8 = slot & 7;
@@ -62,10 +76,19 @@ __global__ __launch_bounds__(256, (MT == 1 ? 3 : (MT == 2 ? 2 : 1))) void w4a16_
     const int nstrips = a.N >> 7;
     const int strip = blockIdx.x % nstrips;
     const int split = blockIdx.x / nstrips;
-    const int chunk = 2 * strip + (slot >> 3);
 
     const int N4 = a.N >> 1;  // 16-byte pieces per packed row
-    const int g_begin = (split * 4 + w) * a.upw;
+    const int g_begin = (split * WAVES + w) * a.upw;
+    const int g_end = (g_begin + a.upw < a.G) ? (g_begin + a.upw) : a.G;
+
+    // per-lane offsets inside the strip (32-bit), everything else is uniform
+    const uint32_t piece_off = (uint32_t)((slot >> 3) * 32 + 4 * c8 + kq);  // 16-byte pieces
+    const uint32_t scale_off = (uint32_t)((slot >> 3) * 64 + 8 * c8);       // halves
+    const u32x4* strip_w = a.B + (size_t)strip * 64;
+    const half_t* strip_s = a.S + (size_t)strip * 128;
+
+    NibbleMagic magic;
+    magic.init();
 
     f4 acc[MT][8];
 #pragma unroll
@@ -73,59 +96,61 @@ __global__ __launch_bounds__(256, (MT == 1 ? 3 : (MT == 2 ? 2 : 1))) void w4a16_
 #pragma unroll
         for (int jb = 0; jb < 8; ++jb) acc[mt][jb] = f4{0.f, 0.f, 0.f, 0.f};
 
-    uint32_t* xs = lds + (size_t)w * (MT * 16) * kXsStride;  // this wave's staging rows
+    uint32_t* xs = lds + (size_t)w * a.xrows * kXsStride;  // this wave's staging rows
+    // MFMA row `slot` of tile mt reads staged row min(16 mt + slot, xrows - 1): rows past M
+    // only feed output rows that are never stored
+    int xrow_of[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        const int r = mt * 16 + slot;
+        xrow_of[mt] = (r < a.xrows ? r : a.xrows - 1) * kXsStride + kq;
+    }
 
     u32x4 wq[8];
-    auto load_weights = [&](int g) {
-        const u32x4* bp = a.B + (size_t)(8 * g) * N4 + chunk * 32 + 4 * c8 + kq;
-#pragma unroll
-        for (int rr = 0; rr < 8; ++rr) wq[rr] = __builtin_nontemporal_load(bp + (size_t)rr * N4);
-    };
-
-    for (int u = 0; u < a.upw; ++u) {
-        const int g = g_begin + u;
-        if (g >= a.G) break;  // wave-uniform
-
-        // ---- activations X[:, 128g .. 128g+127]: issue the loads first ------------
-        u32x4 xv[MT][4];
+    u32x4 sc;
+    u32x4 xv[MT][4];
+    // everything group g needs from memory: activations first (small, they gate the LDS
+    // staging), then scales, then the eight packed rows
+    auto issue_loads = [&](int g) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                const int m = mt * 16 + i * 4 + (lane >> 4);
+                const int m = mt * 16 + i * 4 + kq;
                 xv[mt][i] = u32x4{0u, 0u, 0u, 0u};
                 if (m < a.M)
                     xv[mt][i] = *reinterpret_cast<const u32x4*>(a.X + (size_t)m * a.ldx + 128 * g + 8 * slot);
             }
         }
-
-        // ---- scales of this lane's eight columns --------------------------------
-        u32x4 sc;
         if (!a.per_column) {
-            sc = *reinterpret_cast<const u32x4*>(a.S + (size_t)g * a.N + chunk * 64 + 8 * c8);
+            sc = *reinterpret_cast<const u32x4*>(strip_s + (size_t)g * a.N + scale_off);
         } else {
             uint32_t t[4];
 #pragma unroll
             for (int p = 0; p < 4; ++p) {
-                const int n0 = chunk * 64 + c8 + 8 * (2 * p), n1 = n0 + 8;
+                const int n0 = strip * 128 + (slot >> 3) * 64 + c8 + 8 * (2 * p), n1 = n0 + 8;
                 const uint16_t lo = *reinterpret_cast<const uint16_t*>(a.S + single_scale_pos(n0));
                 const uint16_t hi = *reinterpret_cast<const uint16_t*>(a.S + single_scale_pos(n1));
                 t[p] = (uint32_t)lo | ((uint32_t)hi << 16);
             }
             sc = u32x4{t[0], t[1], t[2], t[3]};
         }
+        const u32x4* rowp = strip_w + (size_t)(8 * g) * N4;  // uniform
+#pragma unroll
+        for (int rr = 0; rr < 8; ++rr) wq[rr] = __builtin_nontemporal_load(rowp + (size_t)rr * N4 + piece_off);
+    };
 
-        // the first group's weights go out behind the (small) activation loads, so
-        // that staging overlaps the weight latency; later groups were prefetched
-        if (u == 0) load_weights(g);
+    if (PF && g_begin < g_end) issue_loads(g_begin);
 
+    for (int g = g_begin; g < g_end; ++g) {  // wave-uniform trip count
+        if (!PF) issue_loads(g);
         // ---- rotate (optionally) and stage the activations in LDS ------------------
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
             for (int i = 0; i < 4; ++i) {
-                {
-                    const int m = mt * 16 + i * 4 + (lane >> 4);
+                const int mrow = mt * 16 + i * 4;
+                if (mrow < a.xrows) {  // uniform
                     u32x4 v = xv[mt][i];
                     if (HAD) {
                         float f[8];
@@ -139,12 +164,12 @@ __global__ __launch_bounds__(256, (MT == 1 ? 3 : (MT == 2 ? 2 : 1))) void w4a16_
 #pragma unroll
                         for (int p = 0; p < 4; ++p) {
                             h2 hv;
-                            hv.x = (half_t)(f[2 * p] * a.had_scale);
-                            hv.y = (half_t)(f[2 * p + 1] * a.had_scale);
+                            hv.x = scaled_to_half(f[2 * p], a.had_scale);
+                            hv.y = scaled_to_half(f[2 * p + 1], a.had_scale);
                             v[p] = h2_to_bits(hv);
                         }
                     }
-                    *reinterpret_cast<u32x4*>(xs + (size_t)m * kXsStride + 4 * slot) = v;
+                    *reinterpret_cast<u32x4*>(xs + (size_t)(mrow + kq) * kXsStride + 4 * slot) = v;
                 }
             }
         }
@@ -154,30 +179,35 @@ __global__ __launch_bounds__(256, (MT == 1 ? 3 : (MT == 2 ? 2 : 1))) void w4a16_
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        // keep the next group's weights in flight while this one is consumed
         u32x4 cur[8];
 #pragma unroll
         for (int rr = 0; rr < 8; ++rr) cur[rr] = wq[rr];
-        if (u + 1 < a.upw && g + 1 < a.G) load_weights(g + 1);
+        const u32x4 sc_cur = sc;
+        // all activation rows this group needs, fetched from LDS before the next group's
+        // loads overwrite the staging registers
+        h8 xa[4][MT];
+#pragma unroll
+        for (int rp = 0; rp < 4; ++rp) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const uint32_t* xr = xs + xrow_of[mt] + 16 * rp;
+                const h2 d0 = bits_to_h2(xr[0]), d1 = bits_to_h2(xr[4]);
+                const h2 d2 = bits_to_h2(xr[8]), d3 = bits_to_h2(xr[12]);
+                xa[rp][mt] = h8{d0.x, d0.y, d1.x, d1.y, d2.x, d2.y, d3.x, d3.y};
+            }
+        }
+        if (PF && g + 1 < g_end) issue_loads(g + 1);
 
         h2 s2[8];
 #pragma unroll
         for (int p = 0; p < 4; ++p) {
-            const h2 pr = bits_to_h2(sc[p]);
+            const h2 pr = bits_to_h2(sc_cur[p]);
             s2[2 * p] = h2{pr.x, pr.x};
             s2[2 * p + 1] = h2{pr.y, pr.y};
         }
 
 #pragma unroll
         for (int rp = 0; rp < 4; ++rp) {
-            h8 xa[MT];
-#pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const uint32_t* xr = xs + (size_t)(mt * 16 + slot) * kXsStride + 16 * rp + kq;
-                const h2 d0 = bits_to_h2(xr[0]), d1 = bits_to_h2(xr[4]);
-                const h2 d2 = bits_to_h2(xr[8]), d3 = bits_to_h2(xr[12]);
-                xa[mt] = h8{d0.x, d0.y, d1.x, d1.y, d2.x, d2.y, d3.x, d3.y};
-            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t q0 = cur[2 * rp][j], q1 = cur[2 * rp + 1][j];
@@ -186,74 +216,76 @@ __global__ __launch_bounds__(256, (MT == 1 ? 3 : (MT == 2 ? 2 : 1))) void w4a16_
                     const uint32_t p0 = blk ? (q0 >> 8) : q0;
                     const uint32_t p1 = blk ? (q1 >> 8) : q1;
                     const h2 sv = s2[2 * j + blk];
-                    const h2 e0 = code_pair_low(p0) * sv, e1 = code_pair_high(p0) * sv;
-                    const h2 e2 = code_pair_low(p1) * sv, e3 = code_pair_high(p1) * sv;
+                    const h2 e0 = magic.pair_low(p0) * sv, e1 = magic.pair_high(p0) * sv;
+                    const h2 e2 = magic.pair_low(p1) * sv, e3 = magic.pair_high(p1) * sv;
                     const h8 bw = h8{e0.x, e0.y, e1.x, e1.y, e2.x, e2.y, e3.x, e3.y};
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
                         acc[mt][2 * j + blk] =
-                            __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt], bw, acc[mt][2 * j + blk], 0, 0, 0);
+                            __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[rp][mt], bw, acc[mt][2 * j + blk], 0, 0, 0);
                 }
             }
         }
     }
 
-    // ---- combine the four waves, then the K splits ---------------------------------
+    // ---- combine the waves (four at a time, fixed order), then the K splits -----------
     // acc[mt][jb][v] on lane l is row m = 16 mt + 4 (l/16) + v, column
     // 128 strip + 64 (slot/8) + 16 (jb/2) + 8 (jb%2) + slot%8.
     float* red = reinterpret_cast<float*>(lds);  // [4 waves][16 rows][128 columns]
+    constexpr int RPT = WAVES / 2;               // output rows covered per pass of the workgroup
+    constexpr int NI = 16 / RPT;                 // passes needed for 16 rows
     const int ncol_lane = 64 * (slot >> 3) + c8;
     const int col_out = tid & 127;
     const int n_out = 128 * strip + col_out;
     for (int mt = 0; mt < MT; ++mt) {
         if (mt * 16 >= a.M) break;
-        __syncthreads();
+        float tot[NI];
 #pragma unroll
-        for (int jb = 0; jb < 8; ++jb) {
+        for (int i = 0; i < NI; ++i) tot[i] = 0.f;
+        for (int round = 0; round < WAVES / 4; ++round) {
+            __syncthreads();
+            if ((w >> 2) == round) {
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int ml = 4 * kq + v;
+                for (int jb = 0; jb < 8; ++jb) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const int ml = 4 * kq + v;
+                        if (mt * 16 + ml < a.M)
+                            red[((w & 3) * 16 + ml) * 128 + ncol_lane + 16 * (jb >> 1) + 8 * (jb & 1)] = acc[mt][jb][v];
+                    }
+                }
+            }
+            __syncthreads();
+#pragma unroll
+            for (int i = 0; i < NI; ++i) {
+                const int ml = (tid >> 7) + RPT * i;
                 if (mt * 16 + ml < a.M)
-                    red[(w * 16 + ml) * 128 + ncol_lane + 16 * (jb >> 1) + 8 * (jb & 1)] = acc[mt][jb][v];
-            }
-        }
-        __syncthreads();
-        for (int ml = tid >> 7; ml < 16; ml += 2) {
-            const int m = mt * 16 + ml;
-            if (m >= a.M) break;
-            const float sum = (red[(0 * 16 + ml) * 128 + col_out] + red[(1 * 16 + ml) * 128 + col_out]) +
+                    tot[i] += (red[(0 * 16 + ml) * 128 + col_out] + red[(1 * 16 + ml) * 128 + col_out]) +
                               (red[(2 * 16 + ml) * 128 + col_out] + red[(3 * 16 + ml) * 128 + col_out]);
-            if (a.splits == 1) {
-                if (a.out_f32)
-                    reinterpret_cast<float*>(a.D)[(size_t)m * a.N + n_out] = sum;
-                else
-                    reinterpret_cast<half_t*>(a.D)[(size_t)m * a.N + n_out] = (half_t)sum;
-            } else {
-                a.partial[((size_t)split * a.M + m) * a.N + n_out] = sum;
             }
         }
-    }
-
-    if (a.splits > 1) {
-        __threadfence();
-        __syncthreads();
-        if (tid == 0) {
-            const int prev = atomicAdd(a.counters + strip, 1);
-            s_last = (prev == a.splits - 1);
-        }
-        __syncthreads();
-        if (s_last) {
-            __threadfence();
-            for (int m = tid >> 7; m < a.M; m += 2) {
-                float sum = 0.f;
-                for (int sp = 0; sp < a.splits; ++sp)
-                    sum += __builtin_nontemporal_load(a.partial + ((size_t)sp * a.M + m) * a.N + n_out);
-                if (a.out_f32)
-                    reinterpret_cast<float*>(a.D)[(size_t)m * a.N + n_out] = sum;
-                else
-                    reinterpret_cast<half_t*>(a.D)[(size_t)m * a.N + n_out] = (half_t)sum;
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int m = mt * 16 + (tid >> 7) + RPT * i;
+            if (m < a.M) {
+                if (a.splits == 1) {
+                    store_out(a, m, n_out, tot[i]);
+                } else {
+                    // fixed point: |v| is clamped to 2^22 (an fp16 result overflows long before),
+                    // so up to 255 contributions fit the 56-bit field
+                    const float v = fminf(fmaxf(tot[i], -kAccumClamp), kAccumClamp);
+                    const long long fixed = __float2ll_rn(v * kAccumScale);
+                    const unsigned long long word = ((unsigned long long)fixed << 8) + 1ull;
+                    unsigned long long* slot_ptr = a.accum + (size_t)m * a.N + n_out;
+                    const unsigned long long old =
+                        __hip_atomic_fetch_add(slot_ptr, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if ((int)(old & 0xffull) == a.splits - 1) {
+                        const long long total = (long long)(old + word) >> 8;
+                        store_out(a, m, n_out, (float)total * (1.0f / kAccumScale));
+                        __hip_atomic_store(slot_ptr, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                }
             }
-            if (tid == 0) a.counters[strip] = 0;
         }
     }
 }
@@ -263,71 +295,111 @@ __global__ __launch_bounds__(256, (MT == 1 ? 3 : (MT == 2 ? 2 : 1))) void w4a16_
 // ---------------------------------------------------------------------------------
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
-int stream_pick_upw(int n, int k) {
+struct StreamPlan {
+    int waves;  // 4, 8 or 16
+    int upw;
+    int splits;
+};
+
+// Heuristic: shapes with enough strips to occupy the chip on their own let one workgroup
+// of 16 waves own a whole strip (no exchange of partial sums); otherwise K is split
+// over workgroups of 4 waves.
+static StreamPlan stream_plan(int m, int n, int k, int upw_override, int waves_override) {
     const int nstrips = n / 128, G = k / 128;
-    int upw = 1;
-    while (upw < 8 && (int64_t)nstrips * ceil_div(G, 4 * upw) > 1024) upw *= 2;
-    return upw;
+    StreamPlan p;
+    p.waves = 4;
+    if (waves_override) p.waves = waves_override;
+    else if (m <= 16 && nstrips >= 192 && G >= 16) p.waves = 16;
+    if (upw_override > 0) {
+        p.upw = upw_override;
+    } else if (p.waves == 16) {
+        p.upw = ceil_div(G, 16);
+        if (p.upw > 8) p.upw = 8;
+    } else {
+        p.upw = 1;
+        while (p.upw < 8 && (int64_t)nstrips * ceil_div(G, p.waves * p.upw) > 1024) p.upw *= 2;
+    }
+    p.splits = ceil_div(G, p.waves * p.upw);
+    while (p.splits > 255) {  // the contribution count has 8 bits
+        p.upw *= 2;
+        p.splits = ceil_div(G, p.waves * p.upw);
+    }
+    return p;
 }
 
-size_t stream_partial_bytes(int m, int n, int k) {
-    // worst case over the possible units-per-wave choices (upw = 1)
+size_t stream_accum_bytes(int m, int n, int k) {
+    // one 64-bit word per output element of a 64-row slab, whenever some plan splits K
     const int G = k / 128;
-    const int splits = ceil_div(G, 4);
-    if (splits <= 1) return 0;
+    if (G <= 4) return 0;
     const int mrows = m < 64 ? m : 64;
-    return (size_t)splits * mrows * n * sizeof(float);
+    return (size_t)mrows * n * sizeof(unsigned long long);
 }
 
-template <int MT, bool HAD>
+template <int MT, bool HAD, int WAVES, bool PF>
 static hipError_t launch_one(const StreamArgs& a, hipStream_t stream) {
-    const size_t stage = (size_t)4 * MT * 16 * kXsStride * 4;
+    const size_t stage = (size_t)WAVES * a.xrows * kXsStride * 4;
     const size_t red = (size_t)4 * 16 * 128 * 4;
     const size_t shmem = stage > red ? stage : red;
+    auto kern = &w4a16_stream_kernel<MT, HAD, WAVES, PF>;
     if (shmem > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&w4a16_stream_kernel<MT, HAD>),
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return e;
     }
     const int grid = (a.N / 128) * a.splits;
-    hipLaunchKernelGGL((w4a16_stream_kernel<MT, HAD>), dim3(grid), dim3(256), shmem, stream, a);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WAVES), shmem, stream, a);
     return hipGetLastError();
 }
 
+template <int MT, bool HAD>
+static hipError_t launch_waves(const StreamArgs& a, int waves, bool pf, hipStream_t stream) {
+    if constexpr (MT == 1) {
+        if (waves == 16) return launch_one<MT, HAD, 16, false>(a, stream);  // 128-register budget: no second weight set
+        if (waves == 8) return pf ? launch_one<MT, HAD, 8, true>(a, stream) : launch_one<MT, HAD, 8, false>(a, stream);
+    }
+    return pf ? launch_one<MT, HAD, 4, true>(a, stream) : launch_one<MT, HAD, 4, false>(a, stream);
+}
+
 // Rows are processed in slabs of at most 64; every slab re-streams the weights.
-int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, int32_t* workspace,
-                  void* scratch, int m, int n, int k, int groups, bool had128, float had_scale, bool out_f32,
-                  int upw_override, hipStream_t stream) {
+// tune: bits 0..7 groups per wave, bits 8..11 waves per workgroup (4/8/16), bit 12 no prefetch;
+// zero fields mean "choose".
+int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, void* accum, int m, int n,
+                  int k, int groups, bool had128, float had_scale, bool out_f32, unsigned tune,
+                  hipStream_t stream) {
     StreamArgs a;
     a.B = reinterpret_cast<const u32x4*>(B);
     a.S = reinterpret_cast<const half_t*>(S);
-    a.partial = reinterpret_cast<float*>(scratch);
-    a.counters = workspace;
+    a.accum = reinterpret_cast<unsigned long long*>(accum);
     a.ldx = lda;
     a.N = n;
     a.K = k;
     a.G = k / 128;
     a.per_column = (groups == 1) ? 1 : 0;
-    a.upw = upw_override > 0 ? upw_override : stream_pick_upw(n, k);
-    a.splits = ceil_div(a.G, 4 * a.upw);
     a.out_f32 = out_f32 ? 1 : 0;
     a.had_scale = had_scale;
+    int waves_override = (int)((tune >> 8) & 0xfu);
+    if (waves_override != 4 && waves_override != 8 && waves_override != 16) waves_override = 0;
     const size_t out_elt = out_f32 ? 4 : 2;
     for (int m0 = 0; m0 < m; m0 += 64) {
         const int mm = (m - m0) < 64 ? (m - m0) : 64;
+        const int mt = mm <= 16 ? 1 : (mm <= 32 ? 2 : 4);
+        const StreamPlan plan = stream_plan(mm, n, k, (int)(tune & 0xffu), mt == 1 ? waves_override : 4);
+        a.upw = plan.upw;
+        a.splits = plan.splits;
         a.M = mm;
+        a.xrows = mt == 1 ? ((mm + 3) / 4) * 4 : mt * 16;
         a.X = reinterpret_cast<const half_t*>(A) + (size_t)m0 * lda;
         a.D = reinterpret_cast<char*>(D) + (size_t)m0 * n * out_elt;
+        const bool pf = !(tune & 0x1000u) && plan.upw > 1 && plan.waves != 16;
         hipError_t e;
-        const int mt = ceil_div(mm, 16);
         if (had128) {
-            if (mt == 1) e = launch_one<1, true>(a, stream);
-            else if (mt == 2) e = launch_one<2, true>(a, stream);
-            else e = launch_one<4, true>(a, stream);
+            if (mt == 1) e = launch_waves<1, true>(a, plan.waves, pf, stream);
+            else if (mt == 2) e = launch_waves<2, true>(a, plan.waves, pf, stream);
+            else e = launch_waves<4, true>(a, plan.waves, pf, stream);
         } else {
-            if (mt == 1) e = launch_one<1, false>(a, stream);
-            else if (mt == 2) e = launch_one<2, false>(a, stream);
-            else e = launch_one<4, false>(a, stream);
+            if (mt == 1) e = launch_waves<1, false>(a, plan.waves, pf, stream);
+            else if (mt == 2) e = launch_waves<2, false>(a, plan.waves, pf, stream);
+            else e = launch_waves<4, false>(a, plan.waves, pf, stream);
         }
         if (e != hipSuccess) return UNIQL_E_LAUNCH;
     }

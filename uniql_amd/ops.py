@@ -25,6 +25,27 @@ def _stream_ptr(device: torch.device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
 
 
+# Zero-in / zero-out accumulator words of the split-K exchange, one buffer per
+# (device, stream): kernels on one stream run in order, so they can share it; work on
+# different streams may overlap and must not.
+_accum_cache: dict = {}
+
+
+def _accumulator(device: torch.device, nbytes: int) -> torch.Tensor:
+    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    buf = _accum_cache.get(key)
+    if buf is None or buf.numel() * 8 < nbytes:
+        buf = torch.zeros(max(nbytes // 8, 1 << 16), dtype=torch.int64, device=device)
+        _accum_cache[key] = buf
+    return buf
+
+
+def reset_accumulators() -> None:
+    """Drops the cached accumulator buffers (they are re-created zeroed).  Only needed
+    after a kernel was aborted half-way, which can leave non-zero words behind."""
+    _accum_cache.clear()
+
+
 def _require_gpu(t: torch.Tensor, name: str) -> None:
     if not t.is_cuda:
         raise RuntimeError(f"{name} must be a GPU tensor (this package has no CPU path)")
@@ -59,15 +80,18 @@ def w4a16_gemm_ex(A: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: 
     out_dtype = torch.float32 if out_f32 else torch.float16
     with torch.cuda.device(dev):
         D = torch.empty((size_m, size_n), dtype=out_dtype, device=dev)
-        need = lib.uniql_w4a16_gemm_scratch_bytes(size_m, size_n, size_k, had_block)
-        scratch = torch.empty(need, dtype=torch.uint8, device=dev) if need else None
+        need_acc = lib.uniql_w4a16_gemm_accum_bytes(size_m, size_n, size_k)
+        accum = _accumulator(dev, need_acc) if need_acc else None
+        need_tmp = lib.uniql_w4a16_gemm_temp_bytes(size_m, size_n, size_k, had_block)
+        temp = torch.empty(need_tmp, dtype=torch.uint8, device=dev) if need_tmp else None
         if out_f32:
             flags |= _capi.F_OUT_F32
         lda = A.stride(0) if size_m > 1 else size_k
         code = lib.uniql_w4a16_gemm(
             A.data_ptr(), lda, B.data_ptr(), s.data_ptr(), D.data_ptr(),
             workspace.data_ptr(), workspace.numel(),
-            scratch.data_ptr() if scratch is not None else None, need,
+            accum.data_ptr() if accum is not None else None, accum.numel() * 8 if accum is not None else 0,
+            temp.data_ptr() if temp is not None else None, need_tmp,
             size_m, size_n, size_k, groups, had_block, float(had_scale), flags, _stream_ptr(dev))
     _capi.check(code, "uniql_w4a16_gemm")
     return D
