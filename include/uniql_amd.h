@@ -35,11 +35,12 @@ enum {
 /* flags of uniql_w4a16_gemm */
 enum {
     UNIQL_F_OUT_F32 = 1 << 0,      /* D is float32 [m, n] instead of fp16 (test hook: the value before the final rounding) */
-    UNIQL_F_FORCE_SKINNY = 1 << 1, /* use the weight-streaming kernel whatever m is */
-    UNIQL_F_FORCE_TILED = 1 << 2,  /* use the prefill (LDS + MFMA tile) kernel whatever m is */
+    UNIQL_F_FORCE_SKINNY = 1 << 1, /* use the weight-streaming kernel (default for m <= 16) whatever m is */
+    UNIQL_F_FORCE_TILED = 1 << 2,  /* use the tiled MFMA kernel (default for m > 16) whatever m is */
     UNIQL_F_TRANSPOSE_OUT = 1 << 3 /* reference's output_transpose; rejected with UNIQL_E_UNSUPPORTED */
-    /* tuning hooks of the streaming kernel, 0 = choose: bits 8..15 K-groups per wavefront,
-       bits 16..19 wavefronts per workgroup (4, 8 or 16), bit 20 disables the register prefetch */
+    /* tuning hooks, 0 = choose.  Streaming kernel: bits 8..15 K-groups per wavefront,
+       bits 16..19 wavefronts per workgroup (4 or 8), bit 20 disables the register prefetch.
+       Tiled kernel: bits 8..15 number of K splits over workgroups. */
 };
 
 int uniql_abi_version(void);
@@ -69,13 +70,14 @@ const char* uniql_status_string(int code);
  *              calls that may run concurrently need separate buffers.  May be NULL
  *              when the size is 0.
  *   temp       device, uniql_w4a16_gemm_temp_bytes(m, n, k, had_block) bytes, contents
- *              irrelevant (rotated activations when had_block is neither 0 nor 128);
+ *              irrelevant (rotated activations whenever the rotation is not fused);
  *              may be NULL when that size is 0
  *   had_block  0: none.  Otherwise the activations are rotated first,
  *              A <- fp16(A . H_had_block * had_scale) on consecutive
  *              had_block-wide pieces of each row: 128 is fused into the
- *              streaming kernel's prologue, any other power of two (<= 32768,
- *              dividing k) runs the transform kernel into `temp` first.
+ *              streaming kernel's prologue (m <= 16); any other power of two
+ *              (<= 32768, dividing k), and 128 for larger m, runs the transform
+ *              kernel into `temp` first.
  *   k % 128 == 0, n % 128 == 0 (the module pads n to 256).
  *
  * Partial sums that meet in `accum` are rounded to multiples of 2^-24 and clamped to

@@ -41,10 +41,11 @@ def test_host_only_entry_points(lib):
     assert b"NULL" in lib.uniql_status_string(-1)
     # one 64-bit word per output element of a (<= 64 row) slab when K can be split
     assert lib.uniql_w4a16_gemm_accum_bytes(1, 4096, 4096) == 4096 * 8
-    assert lib.uniql_w4a16_gemm_accum_bytes(100, 4096, 4096) == 64 * 4096 * 8
+    assert lib.uniql_w4a16_gemm_accum_bytes(100, 4096, 4096) == 100 * 4096 * 8
+    assert lib.uniql_w4a16_gemm_accum_bytes(4096, 4096, 4096) == 64 * 4096 * 8
     assert lib.uniql_w4a16_gemm_accum_bytes(1, 4096, 512) == 0
     assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 8192) == 2 * 8192 * 2
-    assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 128) == 0
+    assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 128) == 2 * 8192 * 2
     assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 0) == 0
 
 

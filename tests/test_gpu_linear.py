@@ -16,7 +16,9 @@ def run_gemm(p, dev, **kw):
     ws = workspace_for(p["n"], dev)
     y = ops.w4a16_gemm_ex(x, b, s, ws, p["m"], p["n"], p["k"], **kw)
     torch.cuda.synchronize()
-    assert int(ws.abs().sum()) == 0, "workspace must be zero again after the call"
+    assert int(ws.abs().sum()) == 0, "workspace must stay zero"
+    for buf in ops._accum_cache.values():
+        assert int(buf.count_nonzero()) == 0, "accumulator words must be zero again after the call"
     return y.cpu().numpy()
 
 
@@ -80,13 +82,69 @@ def test_stream_kernel_llama_shapes(gpu, m, k, n):
     check_layer_output(y16, ref)
 
 
+F_FORCE_SKINNY, F_FORCE_TILED = 2, 4
+
+
 @pytest.mark.parametrize("m", [17, 33, 64, 65, 130])
-def test_stream_kernel_mid_m(gpu, m):
+def test_stream_kernel_forced_for_larger_m(gpu, m):
+    """The streaming kernel walks larger M in slabs of 64 rows (not the default route)."""
     p = make_linear_problem(m, 512, 256, seed=m)
     ref = reference_product(p, exact=True)
-    y32 = run_gemm(p, gpu, out_f32=True)
+    y32 = run_gemm(p, gpu, out_f32=True, flags=F_FORCE_SKINNY)
     assert np.abs(y32 - ref).max() < 2e-4
-    check_layer_output(run_gemm(p, gpu), ref)
+    check_layer_output(run_gemm(p, gpu, flags=F_FORCE_SKINNY), ref)
+
+
+# ------------------------------------------------------------------ prefill shapes (tiled kernel)
+@pytest.mark.parametrize("m", [17, 32, 33, 64, 65, 100, 128, 129, 256, 300])
+@pytest.mark.parametrize("k,n", [(128, 128), (512, 256), (1408, 384)])
+def test_tile_kernel_small_shapes(gpu, m, k, n):
+    p = make_linear_problem(m, k, n, seed=7 * m + k + n)
+    ref = reference_product(p, exact=True)
+    y32 = run_gemm(p, gpu, out_f32=True)
+    assert np.abs(y32 - ref).max() < 2e-4, np.abs(y32 - ref).max()
+    y16 = run_gemm(p, gpu)
+    assert np.array_equal(y16.view(np.uint16), y32.astype(np.float16).view(np.uint16))
+    check_layer_output(y16, ref)
+
+
+@pytest.mark.parametrize("m,k,n", [(256, 4096, 4096), (1024, 4096, 4096), (1024, 4096, 6144), (256, 14336, 4096)])
+def test_tile_kernel_llama_shapes(gpu, m, k, n):
+    p = make_linear_problem(m, k, n, seed=m + k + n)
+    ref = reference_product(p)
+    y16 = run_gemm(p, gpu)
+    check_layer_output(y16, ref)
+
+
+@pytest.mark.parametrize("m", [1, 5, 16])
+def test_tile_kernel_forced_for_small_m(gpu, m):
+    p = make_linear_problem(m, 640, 256, seed=m + 3)
+    ref = reference_product(p, exact=True)
+    y32 = run_gemm(p, gpu, out_f32=True, flags=F_FORCE_TILED)
+    assert np.abs(y32 - ref).max() < 2e-4
+
+
+@pytest.mark.parametrize("splits", [1, 2, 3, 11])
+def test_tile_kernel_k_splits(gpu, splits):
+    p = make_linear_problem(40, 1408, 256, seed=splits)        # 11 groups
+    ref = reference_product(p, exact=True)
+    y32 = run_gemm(p, gpu, out_f32=True, flags=splits << 8)
+    assert np.abs(y32 - ref).max() < 2e-4
+    again = run_gemm(p, gpu, out_f32=True, flags=splits << 8)
+    assert np.array_equal(y32, again)                          # integer accumulation: order-independent
+
+
+def test_tile_kernel_per_column_and_stride(gpu):
+    from uniql_amd import ops
+    p = make_linear_problem(48, 384, 256, seed=21, per_column=True)
+    ref = reference_product(p, exact=True)
+    assert np.abs(run_gemm(p, gpu, out_f32=True) - ref).max() < 2e-4
+    p = make_linear_problem(40, 256, 256, seed=22)
+    x, b, s = to_gpu(p, gpu)
+    big = torch.zeros(40, 512, dtype=torch.float16, device=gpu)
+    big[:, :256] = x
+    y = ops.w4a16_gemm_ex(big[:, :256], b, s, workspace_for(256, gpu), 40, 256, 256).cpu().numpy()
+    check_layer_output(y, reference_product(p))
 
 
 @pytest.mark.parametrize("upw", [1, 2, 4, 8])
@@ -124,7 +182,7 @@ def test_row_stride(gpu):
 
 
 # ------------------------------------------------------------------ fused rotation
-@pytest.mark.parametrize("m", [1, 5, 16, 40])
+@pytest.mark.parametrize("m", [1, 5, 16, 40, 200])
 def test_fused_blockwise_hadamard(gpu, m):
     k, n = 1536, 256           # 12 blocks of 128: not a power of two overall
     p = make_linear_problem(m, k, n, seed=m + 40)

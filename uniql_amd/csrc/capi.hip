@@ -7,6 +7,9 @@ int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void
                   int k, int groups, bool had128, float had_scale, bool out_f32, unsigned tune,
                   hipStream_t stream);
 size_t stream_accum_bytes(int m, int n, int k);
+int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, void* accum, size_t accum_bytes,
+                int m, int n, int k, int groups, bool out_f32, unsigned tune, hipStream_t stream);
+size_t tile_accum_bytes(int m, int n, int k);
 int dequant_launch(const void* B, const void* S, void* W, uint8_t* codes, int n, int k, int groups,
                    hipStream_t stream);
 int embedding_launch(const int64_t* ids, int64_t ntokens, const void* weight, const void* scales, void* out,
@@ -45,14 +48,21 @@ const char* uniql_status_string(int code) {
     }
 }
 
+// rows up to this many take the weight-streaming kernel, more take the tiled one
+static constexpr int kStreamMaxM = 16;
+
 size_t uniql_w4a16_gemm_accum_bytes(int m, int n, int k) {
-    if (m <= 0 || n <= 0 || k <= 0) return 0;
-    return round256(stream_accum_bytes(m, n, k));
+    if (m <= 0 || n <= 0 || k <= 0 || n % 128 != 0 || k % 128 != 0) return 0;
+    // enough for either kernel, so that the forcing flags never need a bigger buffer
+    const size_t a = stream_accum_bytes(m, n, k), b = tile_accum_bytes(m, n, k);
+    return round256(a > b ? a : b);
 }
 
 size_t uniql_w4a16_gemm_temp_bytes(int m, int n, int k, int had_block) {
     if (m <= 0 || n <= 0 || k <= 0) return 0;
-    if (had_block != 0 && had_block != 128) return round256((size_t)m * k * sizeof(half_t));
+    // rotated activations: every block width except the 128 fused into the streaming kernel,
+    // and 128 too once the tiled kernel may take the call
+    if (had_block != 0) return round256((size_t)m * k * sizeof(half_t));
     return 0;
 }
 
@@ -76,9 +86,13 @@ int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, v
     if ((accum && !aligned16(accum)) || (temp && !aligned16(temp))) return UNIQL_E_ALIGN;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 
+    bool use_stream = m <= kStreamMaxM;
+    if (flags & UNIQL_F_FORCE_SKINNY) use_stream = true;
+    if (flags & UNIQL_F_FORCE_TILED) use_stream = false;
+
     const void* Ain = A;
     int64_t ld = lda;
-    const bool had128 = (had_block == 128);
+    const bool had128 = (had_block == 128) && use_stream;
     if (had_block != 0 && !had128) {
         // rotate into the temporary buffer, then run the plain product on it
         if (lda != k) {
@@ -96,8 +110,11 @@ int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, v
         ld = k;
     }
     const unsigned tune = flags >> 8;  // tuning fields, see the header
-    return stream_launch(Ain, ld, B, S, D, accum, m, n, k, groups, had128, had_scale,
-                         (flags & UNIQL_F_OUT_F32) != 0, tune, st);
+    if (use_stream)
+        return stream_launch(Ain, ld, B, S, D, accum, m, n, k, groups, had128, had_scale,
+                             (flags & UNIQL_F_OUT_F32) != 0, tune, st);
+    return tile_launch(Ain, ld, B, S, D, accum, accum_bytes, m, n, k, groups, (flags & UNIQL_F_OUT_F32) != 0, tune,
+                       st);
 }
 
 int uniql_w4a16_dequant(const void* B, const void* S, void* W, uint8_t* codes, int n, int k, int groups,
