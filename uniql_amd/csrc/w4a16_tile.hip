@@ -1,29 +1,42 @@
 // Tiled W4A16 kernel for M > 16 (prefill): D[M,N] = X[M,K] . dequant(B)[K,N].
 //
-// A workgroup of four wavefronts owns a (16 MTILES) x 128 output tile and a range of
-// 128-wide K groups.  The packed weights never touch LDS: as in the streaming kernel,
-// each wave fetches 16-byte pieces in the lane order that makes the registers the B
-// operand of v_mfma_f32_16x16x32_f16 (lane = column slot + 16 * K quarter), expands them
-// to fp16 (code-8)*scale in registers and feeds MFMA directly.  The four waves split
-// every K group between them (wave w takes the two packed rows 2w, 2w+1 = 32 K values),
-// so every weight of the tile is expanded exactly once per workgroup.
+// A workgroup of four wavefronts owns a (32 MT) x 128 output tile (MT = 1, 2 or 4) and a
+// range of 128-wide K groups.  The four waves split K: of the eight packed rows (16 K
+// values each) of a group, wave w takes rows w and w + 4 and accumulates the WHOLE tile
+// for them with v_mfma_f32_32x32x16_f16, so every weight of the tile is expanded to fp16
+// (code-8)*scale exactly once per workgroup.  The partial tiles of the four waves are
+// added through LDS at the end.
 //
-// The activations are the A operand.  The X tile of a K group (rows x 128 halves) is
-// loaded by the whole workgroup with coalesced 16-byte loads into LDS (double buffered,
-// row stride 68 dwords so that the 64 lanes of an operand read hit 64 distinct banks);
-// each wave reads the 32-K slice it needs for all its 16-row M tiles.  Global loads
-// for group g+1 (X tile, packed rows, scales) are issued before the MFMAs of group g.
+// Operand layout.  A 16-byte piece (c8, kq) of a packed row holds, in 32-bit word j,
+// K rows {2kq, 2kq+1, 2kq+8, 2kq+9} of columns 16j + c8 and 16j + 8 + c8.  Lane
+//     l = s + 32 h,  s = c8 + 8 ch + 16 jl      (ch: 64-column chunk of the strip)
+// reads words 2jl, 2jl+1 of the pieces kq = 2h and 2h+1 and builds four B operands
+// (jo, blk): column 64 ch + 16 (2jl + jo) + 8 blk + c8, K values {4h..4h+3, 4h+8..4h+11}.
+// The A operand of a 32-row M tile is row l % 32 of X with the same eight K values
+// (two 8-byte LDS reads).
 //
-// At the end the four waves' accumulators meet in LDS.  When K is also split over
-// workgroups (grid.z > 1) the tile goes through the same 64-bit fixed-point
+// Everything a group needs travels global -> LDS with global_load_lds_dwordx4 (no staging
+// registers) into a ring of three stages; the loads of group g+2 are issued when group g
+// starts computing.  A stage holds
+//   * the X tile, 256 bytes per row, unpadded: 16-byte segment sg of row r sits at position
+//     sg ^ (r % 16);
+//   * per wave, its two packed rows of the strip (2 x 1 KiB): piece (c8, ch, kq) at position
+//     c8 + 8 ch + 16 kq, so a half-wave's 8-byte reads sweep all 64 banks;
+//   * per wave, the 256 bytes of scales of the strip.
+// vmcnt is counted by hand: every stage issues exactly kStageOps LDS-DMA operations per
+// wave and nothing else uses the counter inside the loop.
+//
+// When K is also split over workgroups the tile goes through the same 64-bit fixed-point
 // sum|count words as the streaming kernel.
 #include "common.hpp"
 
 namespace uniql {
 
-constexpr int kTileXsStride = 68;            // dwords per staged X row (64 + 4)
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
 constexpr float kTileAccumScale = 16777216.0f;  // 2^24
 constexpr float kTileAccumClamp = 4194304.0f;   // 2^22
+constexpr int kRing = 3;
 
 struct TileArgs {
     const u32x4* B;
@@ -37,22 +50,48 @@ struct TileArgs {
     int per_column;
     int gps;          // K groups per split
     int splits;
-    int mblocks;      // ceil(M / (16 MTILES))
+    int mblocks;      // ceil(M / (32 MT))
     int out_f32;
 };
 
-template <int MTILES>
+typedef const __attribute__((address_space(1))) void* gptr_t;
+typedef __attribute__((address_space(3))) void* lptr_t;
+
+// s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding)
+#define UNIQL_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
+
+template <int MT>
+struct TileLds {
+    static constexpr int kRows = 32 * MT;
+    static constexpr int kXDwords = kRows * 64;        // X tile
+    static constexpr int kBDwords = 4 * 2 * 256;       // 4 waves x 2 packed rows x 1 KiB
+    static constexpr int kSDwords = 4 * 64;            // 4 waves x 256 bytes of scales
+    static constexpr int kStageDwords = kXDwords + kBDwords + kSDwords;
+    static constexpr size_t kRingBytes = (size_t)kRing * kStageDwords * 4;
+    static constexpr size_t kRedBytes = (size_t)4 * 32 * 128 * 4;  // 4 waves x one 32-row M tile, fp32
+    static constexpr size_t kBytes = kRingBytes > kRedBytes ? kRingBytes : kRedBytes;
+};
+
+template <int MT>
 __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
-    constexpr int ROWS = 16 * MTILES;
-    constexpr int BUF_DWORDS = ROWS * kTileXsStride;
+    using L = TileLds<MT>;
+    constexpr int ROWS = L::kRows;
+    constexpr int kXOps = ROWS / 16;        // X DMA instructions per wave and stage (4 rows each)
+    constexpr int kStageOps = kXOps + 3;    // + two packed rows + scales
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int slot = lane & 15;
-    const int kq = lane >> 4;
-    const int c8 = slot & 7;
+    // MFMA view of the lane
+    const int s = lane & 31;
+    const int h = lane >> 5;
+    const int c8 = s & 7;
+    const int ch = (s >> 3) & 1;
+    const int jl = s >> 4;
+    // DMA view of the lane (16 lanes per X row; piece gather for the packed rows)
+    const int dslot = lane & 15;
+    const int dkq = lane >> 4;
 
     // tile coordinates: strips vary fastest so that neighbouring workgroups share X rows
     const int nstrips = a.N >> 7;
@@ -66,127 +105,175 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     const int N4 = a.N >> 1;
     const int g_begin = split * a.gps;
     const int g_end = (g_begin + a.gps < a.G) ? (g_begin + a.gps) : a.G;
+    const int ngroups = g_end - g_begin;
 
-    const uint32_t piece_off = (uint32_t)((slot >> 3) * 32 + 4 * c8 + kq);
-    const uint32_t scale_off = (uint32_t)((slot >> 3) * 64 + 8 * c8);
-    const u32x4* strip_w = a.B + (size_t)strip * 64 + (size_t)(2 * w) * N4;  // this wave's two rows of a group
-    const half_t* strip_s = a.S + (size_t)strip * 128;
+    // packed rows w and w + 4 of every group; DMA lane (c8', ch', kq') fetches piece 32 ch' + 4 c8' + kq'
+    const uint32_t piece_off = (uint32_t)((dslot >> 3) * 32 + 4 * (dslot & 7) + dkq);
+    const u32x4* strip_w = a.B + (size_t)strip * 64 + (size_t)w * N4 + piece_off;
+    // scales: lanes 0..15 fetch the 16 pieces (8 halves each) of the strip's 128 columns
+    const half_t* strip_s = a.S + (size_t)strip * 128 + 8 * dslot;
 
-    // cooperative X tile load: thread t covers row (t / 16) + 16 p, 16-byte segment t % 16
-    const int xr_row = tid >> 4;
-    const int xr_seg = tid & 15;
+    // X tile: wave w brings rows [kXOps 4 w, kXOps 4 (w+1)); one DMA instruction covers 4 rows
+    // (64 lanes x 16 bytes, contiguous in LDS).  Lane l lands at row l/16, position l%16, so
+    // it must fetch segment (l % 16) ^ (row % 16) of its row.
+    const half_t* xsrc[kXOps];
+#pragma unroll
+    for (int i = 0; i < kXOps; ++i) {
+        const int row = kXOps * 4 * w + 4 * i + dkq;
+        const int seg = dslot ^ (row & 15);
+        const int m = m0 + row;
+        const int mc = m < a.M ? m : a.M - 1;  // rows past M re-read the last row: never stored
+        xsrc[i] = a.X + (size_t)mc * a.ldx + 8 * seg;
+    }
 
     NibbleMagic magic;
     magic.init();
 
-    f4 acc[MTILES][8];
+    f16 acc[MT][4];
 #pragma unroll
-    for (int mt = 0; mt < MTILES; ++mt)
+    for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int jb = 0; jb < 8; ++jb) acc[mt][jb] = f4{0.f, 0.f, 0.f, 0.f};
+        for (int op = 0; op < 4; ++op)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[mt][op][v] = 0.f;
 
-    u32x4 xv[MTILES];
-    u32x4 wq[2];
-    u32x4 sc;
-    auto issue_loads = [&](int g) {
+    // per-column scales do not depend on the group: fetch them once, into registers
+    u32x2 sc_fixed = u32x2{0u, 0u};
+    if (a.per_column) {
+        uint32_t t[2];
 #pragma unroll
-        for (int p = 0; p < MTILES; ++p) {
-            const int m = m0 + xr_row + 16 * p;
-            xv[p] = u32x4{0u, 0u, 0u, 0u};
-            if (m < a.M) xv[p] = *reinterpret_cast<const u32x4*>(a.X + (size_t)m * a.ldx + 128 * g + 8 * xr_seg);
+        for (int jo = 0; jo < 2; ++jo) {
+            const int n0 = strip * 128 + 64 * ch + 16 * (2 * jl + jo) + c8, n1 = n0 + 8;
+            const uint16_t lo = *reinterpret_cast<const uint16_t*>(a.S + single_scale_pos(n0));
+            const uint16_t hi = *reinterpret_cast<const uint16_t*>(a.S + single_scale_pos(n1));
+            t[jo] = (uint32_t)lo | ((uint32_t)hi << 16);
         }
-        if (!a.per_column) {
-            sc = *reinterpret_cast<const u32x4*>(strip_s + (size_t)g * a.N + scale_off);
+        sc_fixed = u32x2{t[0], t[1]};
+        UNIQL_WAIT_VMCNT(0);  // keep the hand count below exact: nothing of this stays outstanding
+    }
+
+    // One of the kStageOps LDS-DMA operations that bring group g into ring slot `ring`:
+    // idx < kXOps: four X rows; kXOps, kXOps + 1: the two packed rows; kXOps + 2: scales.
+    // The operations of a stage are spread between the MFMA blocks of the previous stage, so
+    // the wave never sits behind a full address queue (the tile needs ~60% of the CU's
+    // 64 B/clk vector-memory path).
+    auto issue_piece = [&](int g, int ring, int idx) {
+        uint32_t* stage = lds + ring * L::kStageDwords;
+        if (idx < kXOps) {
+            uint32_t* xbuf = stage + (kXOps * 4 * w) * 64;  // this wave's X rows
+            __builtin_amdgcn_global_load_lds((gptr_t)(xsrc[idx] + 128 * g), (lptr_t)(xbuf + idx * 256), 16, 0, 0);
+        } else if (idx < kXOps + 2) {
+            uint32_t* bbuf = stage + L::kXDwords + w * 512 + (idx - kXOps) * 256;
+            const u32x4* rowp = strip_w + (size_t)(8 * g + 4 * (idx - kXOps)) * N4;
+            __builtin_amdgcn_global_load_lds((gptr_t)rowp, (lptr_t)bbuf, 16, 0, 0);
         } else {
-            uint32_t t[4];
-#pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                const int n0 = strip * 128 + (slot >> 3) * 64 + c8 + 8 * (2 * p), n1 = n0 + 8;
-                const uint16_t lo = *reinterpret_cast<const uint16_t*>(a.S + single_scale_pos(n0));
-                const uint16_t hi = *reinterpret_cast<const uint16_t*>(a.S + single_scale_pos(n1));
-                t[p] = (uint32_t)lo | ((uint32_t)hi << 16);
-            }
-            sc = u32x4{t[0], t[1], t[2], t[3]};
+            // scales of the group (row 0 in per-column mode, unused then)
+            uint32_t* sbuf = stage + L::kXDwords + L::kBDwords + w * 64;
+            const half_t* ssrc = strip_s + (a.per_column ? (size_t)0 : (size_t)g * a.N);
+            if (dkq == 0) __builtin_amdgcn_global_load_lds((gptr_t)ssrc, (lptr_t)sbuf, 16, 0, 0);
         }
-        const u32x4* rowp = strip_w + (size_t)(8 * g) * N4;
-        wq[0] = rowp[piece_off];
-        wq[1] = rowp[(size_t)N4 + piece_off];
     };
-    auto stage_x = [&](int buf) {
-        uint32_t* dst = lds + buf * BUF_DWORDS;
+    auto issue_stage = [&](int g, int ring) {
 #pragma unroll
-        for (int p = 0; p < MTILES; ++p)
-            *reinterpret_cast<u32x4*>(dst + (xr_row + 16 * p) * kTileXsStride + 4 * xr_seg) = xv[p];
+        for (int idx = 0; idx < kStageOps; ++idx) issue_piece(g, ring, idx);
     };
 
-    if (g_begin < g_end) {
-        issue_loads(g_begin);
-        stage_x(0);
+    // LDS read offsets (dwords).  X: row s of an M tile, packed row w + 4 t -> segments
+    // 2 (w + 4t) and 2 (w + 4t) + 1, K half h = dwords 2h, 2h+1 of the segment.
+    int xoff[2][2];
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+        for (int x = 0; x < 2; ++x) xoff[t][x] = s * 64 + (((2 * (w + 4 * t) + x) ^ (s & 15)) << 2) + 2 * h;
+    const int boff = (c8 + 8 * ch + 32 * h) * 4 + 2 * jl;  // piece kq = 2h, words 2jl, 2jl+1; kq = 2h+1 is 64 dwords on
+    const int soff = (8 * ch + c8) * 4 + 2 * jl;
+
+    // next_g >= 0: also issue the loads of group next_g into slot next_ring, between the MFMA blocks
+    auto compute_stage = [&](int ring, int next_g, int next_ring) {
+        const uint32_t* stage = lds + ring * L::kStageDwords;
+        const uint32_t* bbuf = stage + L::kXDwords + w * 512;
+        u32x2 sc_cur = sc_fixed;
+        if (!a.per_column)
+            sc_cur = *reinterpret_cast<const u32x2*>(stage + L::kXDwords + L::kBDwords + w * 64 + soff);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            const u32x2 p0 = *reinterpret_cast<const u32x2*>(bbuf + t * 256 + boff);
+            const u32x2 p1 = *reinterpret_cast<const u32x2*>(bbuf + t * 256 + boff + 64);
+            h8 xa[MT];
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+                const u32x2 lo = *reinterpret_cast<const u32x2*>(stage + mt * 2048 + xoff[t][0]);
+                const u32x2 hi = *reinterpret_cast<const u32x2*>(stage + mt * 2048 + xoff[t][1]);
+                const h2 d0 = bits_to_h2(lo.x), d1 = bits_to_h2(lo.y), d2 = bits_to_h2(hi.x), d3 = bits_to_h2(hi.y);
+                xa[mt] = h8{d0.x, d0.y, d1.x, d1.y, d2.x, d2.y, d3.x, d3.y};
+            }
+#pragma unroll
+            for (int jo = 0; jo < 2; ++jo) {
+                const h2 pr = bits_to_h2(sc_cur[jo]);
+#pragma unroll
+                for (int blk = 0; blk < 2; ++blk) {
+                    const uint32_t q0 = blk ? (p0[jo] >> 8) : p0[jo];
+                    const uint32_t q1 = blk ? (p1[jo] >> 8) : p1[jo];
+                    const h2 sv = blk ? h2{pr.y, pr.y} : h2{pr.x, pr.x};
+                    // K order of the operand: 4h, 4h+1 | 4h+2, 4h+3 | 4h+8, 4h+9 | 4h+10, 4h+11
+                    const h2 e0 = magic.pair_low(q0) * sv, e1 = magic.pair_low(q1) * sv;
+                    const h2 e2 = magic.pair_high(q0) * sv, e3 = magic.pair_high(q1) * sv;
+                    const h8 bw = h8{e0.x, e0.y, e1.x, e1.y, e2.x, e2.y, e3.x, e3.y};
+#pragma unroll
+                    for (int mt = 0; mt < MT; ++mt)
+                        acc[mt][2 * jo + blk] =
+                            __builtin_amdgcn_mfma_f32_32x32x16_f16(xa[mt], bw, acc[mt][2 * jo + blk], 0, 0, 0);
+                    if (next_g >= 0) {  // uniform
+                        const int block = 4 * t + 2 * jo + blk;  // 0..7
+#pragma unroll
+                        for (int idx = block; idx < kStageOps; idx += 8) issue_piece(next_g, next_ring, idx);
+                    }
+                }
+            }
+        }
+    };
+
+    // ---- software pipeline over the K groups ----------------------------------------------
+    if (ngroups > 0) issue_stage(g_begin, 0);
+    if (ngroups > 1) issue_stage(g_begin + 1, 1);
+    int ring = 0;
+    for (int it = 0; it < ngroups; ++it) {
+        // stage it+1 may stay in flight; stage it has landed once only that one is outstanding
+        if (it + 1 < ngroups) UNIQL_WAIT_VMCNT(kStageOps);
+        else UNIQL_WAIT_VMCNT(0);
+        __builtin_amdgcn_s_barrier();  // all waves' parts of stage `it` are in LDS, and everyone has
+                                       // finished reading the slot that is refilled next
+        const int refill = ring == 0 ? kRing - 1 : ring - 1;  // == (it + 2) % kRing
+        compute_stage(ring, it + 2 < ngroups ? g_begin + it + 2 : -1, refill);
+        ring = ring + 1 == kRing ? 0 : ring + 1;
     }
     __syncthreads();
 
-    for (int g = g_begin; g < g_end; ++g) {
-        const int buf = (g - g_begin) & 1;
-        const u32x4 cur0 = wq[0], cur1 = wq[1];
-        const u32x4 sc_cur = sc;
-        if (g + 1 < g_end) issue_loads(g + 1);
-
-        // A operands of this wave's 32-K slice, all M tiles
-        const uint32_t* xs = lds + buf * BUF_DWORDS + 16 * w + kq;
-        h8 xa[MTILES];
-#pragma unroll
-        for (int mt = 0; mt < MTILES; ++mt) {
-            const uint32_t* xr = xs + (mt * 16 + slot) * kTileXsStride;
-            const h2 d0 = bits_to_h2(xr[0]), d1 = bits_to_h2(xr[4]);
-            const h2 d2 = bits_to_h2(xr[8]), d3 = bits_to_h2(xr[12]);
-            xa[mt] = h8{d0.x, d0.y, d1.x, d1.y, d2.x, d2.y, d3.x, d3.y};
-        }
-
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const uint32_t q0 = cur0[j], q1 = cur1[j];
-            const h2 pr = bits_to_h2(sc_cur[j]);
-#pragma unroll
-            for (int blk = 0; blk < 2; ++blk) {
-                const uint32_t p0 = blk ? (q0 >> 8) : q0;
-                const uint32_t p1 = blk ? (q1 >> 8) : q1;
-                const h2 sv = blk ? h2{pr.y, pr.y} : h2{pr.x, pr.x};
-                const h2 e0 = magic.pair_low(p0) * sv, e1 = magic.pair_high(p0) * sv;
-                const h2 e2 = magic.pair_low(p1) * sv, e3 = magic.pair_high(p1) * sv;
-                const h8 bw = h8{e0.x, e0.y, e1.x, e1.y, e2.x, e2.y, e3.x, e3.y};
-#pragma unroll
-                for (int mt = 0; mt < MTILES; ++mt)
-                    acc[mt][2 * j + blk] =
-                        __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[mt], bw, acc[mt][2 * j + blk], 0, 0, 0);
-            }
-        }
-
-        if (g + 1 < g_end) stage_x(buf ^ 1);
-        __syncthreads();
-    }
-
-    // ---- combine the four waves, one 16-row M tile at a time -------------------------------
-    float* red = reinterpret_cast<float*>(lds);  // [4 waves][16 rows][128 columns]
-    const int ncol_lane = 64 * (slot >> 3) + c8;
+    // ---- add the four waves' partial tiles, one 32-row M tile at a time ---------------------
+    // acc[mt][2 jo + blk][v] on lane l: row 32 mt + 8 (v / 4) + 4 h + v % 4,
+    // column 64 ch + 16 (2 jl + jo) + 8 blk + c8 of the strip.
+    float* red = reinterpret_cast<float*>(lds);  // [4 waves][32 rows][128 columns]
     const int col_out = tid & 127;
     const int n_out = 128 * strip + col_out;
 #pragma unroll
-    for (int mt = 0; mt < MTILES; ++mt) {
-        if (m0 + mt * 16 < a.M) {  // uniform
+    for (int mt = 0; mt < MT; ++mt) {
+        if (m0 + mt * 32 < a.M) {  // uniform
             if (mt > 0) __syncthreads();
 #pragma unroll
-            for (int jb = 0; jb < 8; ++jb)
+            for (int op = 0; op < 4; ++op) {
+                const int ncol = 64 * ch + 16 * (2 * jl + (op >> 1)) + 8 * (op & 1) + c8;
 #pragma unroll
-                for (int v = 0; v < 4; ++v)
-                    red[(w * 16 + 4 * kq + v) * 128 + ncol_lane + 16 * (jb >> 1) + 8 * (jb & 1)] = acc[mt][jb][v];
+                for (int v = 0; v < 16; ++v)
+                    red[(w * 32 + 8 * (v >> 2) + 4 * h + (v & 3)) * 128 + ncol] = acc[mt][op][v];
+            }
             __syncthreads();
 #pragma unroll
-            for (int i = 0; i < 8; ++i) {
+            for (int i = 0; i < 16; ++i) {
                 const int ml = (tid >> 7) + 2 * i;
-                const int m = m0 + mt * 16 + ml;
+                const int m = m0 + mt * 32 + ml;
                 if (m < a.M) {
-                    const float sum = (red[(0 * 16 + ml) * 128 + col_out] + red[(1 * 16 + ml) * 128 + col_out]) +
-                                      (red[(2 * 16 + ml) * 128 + col_out] + red[(3 * 16 + ml) * 128 + col_out]);
+                    const float sum = (red[(0 * 32 + ml) * 128 + col_out] + red[(1 * 32 + ml) * 128 + col_out]) +
+                                      (red[(2 * 32 + ml) * 128 + col_out] + red[(3 * 32 + ml) * 128 + col_out]);
                     float outv = sum;
                     bool emit = true;
                     unsigned long long* slot_ptr = nullptr;
@@ -228,9 +315,9 @@ size_t tile_accum_bytes(int m, int n, int k) {
 
 static TilePlan tile_plan(int m, int n, int k, int splits_override) {
     TilePlan p;
-    p.mtiles = m <= 32 ? 2 : (m <= 64 ? 4 : 8);
+    p.mtiles = m <= 32 ? 1 : (m <= 64 ? 2 : 4);  // 32-row M tiles per workgroup
     const int G = k / 128;
-    const int tiles = (n / 128) * ceil_div_i(m, 16 * p.mtiles);
+    const int tiles = (n / 128) * ceil_div_i(m, 32 * p.mtiles);
     int splits = 1;
     if (splits_override > 0) {
         splits = splits_override;
@@ -245,12 +332,10 @@ static TilePlan tile_plan(int m, int n, int k, int splits_override) {
     return p;
 }
 
-template <int MTILES>
+template <int MT>
 static hipError_t tile_launch_one(const TileArgs& a, int grid, hipStream_t stream) {
-    const size_t stage = (size_t)2 * 16 * MTILES * kTileXsStride * 4;
-    const size_t red = (size_t)4 * 16 * 128 * 4;
-    const size_t shmem = stage > red ? stage : red;
-    auto kern = &w4a16_tile_kernel<MTILES>;
+    const size_t shmem = TileLds<MT>::kBytes;
+    auto kern = &w4a16_tile_kernel<MT>;
     if (shmem > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -280,14 +365,14 @@ int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* 
     a.per_column = (groups == 1) ? 1 : 0;
     a.gps = plan.gps;
     a.splits = plan.splits;
-    a.mblocks = ceil_div_i(m, 16 * plan.mtiles);
+    a.mblocks = ceil_div_i(m, 32 * plan.mtiles);
     a.out_f32 = out_f32 ? 1 : 0;
     const int64_t grid = (int64_t)(n / 128) * a.mblocks * a.splits;
     if (grid > 0x7fffffffLL) return UNIQL_E_SHAPE;
     hipError_t e;
-    if (plan.mtiles == 2) e = tile_launch_one<2>(a, (int)grid, stream);
-    else if (plan.mtiles == 4) e = tile_launch_one<4>(a, (int)grid, stream);
-    else e = tile_launch_one<8>(a, (int)grid, stream);
+    if (plan.mtiles == 1) e = tile_launch_one<1>(a, (int)grid, stream);
+    else if (plan.mtiles == 2) e = tile_launch_one<2>(a, (int)grid, stream);
+    else e = tile_launch_one<4>(a, (int)grid, stream);
     return e == hipSuccess ? UNIQL_OK : UNIQL_E_LAUNCH;
 }
 
