@@ -16,8 +16,9 @@
 // (two 8-byte LDS reads).
 //
 // Everything a group needs travels global -> LDS with global_load_lds_dwordx4 (no staging
-// registers) into a ring of three stages; the loads of group g+2 are issued when group g
-// starts computing.  A stage holds
+// registers) into a ring of three stages; the loads of group g+2 are issued while group g
+// is multiplied, and the operands of group g+1 are read from LDS into a second register set
+// during the second half of group g.  A stage holds
 //   * the X tile, 256 bytes per row, unpadded: 16-byte segment sg of row r sits at position
 //     sg ^ (r % 16);
 //   * per wave, its two packed rows of the strip (2 x 1 KiB): piece (c8, ch, kq) at position
@@ -68,7 +69,7 @@ struct TileLds {
     static constexpr int kSDwords = 4 * 64;            // 4 waves x 256 bytes of scales
     static constexpr int kStageDwords = kXDwords + kBDwords + kSDwords;
     static constexpr size_t kRingBytes = (size_t)kRing * kStageDwords * 4;
-    static constexpr size_t kRedBytes = (size_t)4 * 32 * 128 * 4;  // 4 waves x one 32-row M tile, fp32
+    static constexpr size_t kRedBytes = (size_t)4 * 32 * 132 * 4;  // 4 waves x one 32-row M tile, fp32, padded rows
     static constexpr size_t kBytes = kRingBytes > kRedBytes ? kRingBytes : kRedBytes;
 };
 
@@ -109,21 +110,21 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
 
     // packed rows w and w + 4 of every group; DMA lane (c8', ch', kq') fetches piece 32 ch' + 4 c8' + kq'
     const uint32_t piece_off = (uint32_t)((dslot >> 3) * 32 + 4 * (dslot & 7) + dkq);
-    const u32x4* strip_w = a.B + (size_t)strip * 64 + (size_t)w * N4 + piece_off;
+    const u32x4* strip_w = a.B + (size_t)strip * 64 + (size_t)w * N4;  // uniform; the lane adds piece_off
     // scales: lanes 0..15 fetch the 16 pieces (8 halves each) of the strip's 128 columns
-    const half_t* strip_s = a.S + (size_t)strip * 128 + 8 * dslot;
+    const half_t* strip_s = a.S + (size_t)strip * 128;  // uniform; the lane adds 8 * dslot
 
     // X tile: wave w brings rows [kXOps 4 w, kXOps 4 (w+1)); one DMA instruction covers 4 rows
     // (64 lanes x 16 bytes, contiguous in LDS).  Lane l lands at row l/16, position l%16, so
     // it must fetch segment (l % 16) ^ (row % 16) of its row.
-    const half_t* xsrc[kXOps];
+    uint32_t xsrc[kXOps];  // byte offsets from X + 128 g (uniform): scalar base + 32-bit lane offset addressing
 #pragma unroll
     for (int i = 0; i < kXOps; ++i) {
         const int row = kXOps * 4 * w + 4 * i + dkq;
         const int seg = dslot ^ (row & 15);
         const int m = m0 + row;
         const int mc = m < a.M ? m : a.M - 1;  // rows past M re-read the last row: never stored
-        xsrc[i] = a.X + (size_t)mc * a.ldx + 8 * seg;
+        xsrc[i] = (uint32_t)(((size_t)mc * a.ldx + 8 * seg) * sizeof(half_t));
     }
 
     NibbleMagic magic;
@@ -157,23 +158,24 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     // The operations of a stage are spread between the MFMA blocks of the previous stage, so
     // the wave never sits behind a full address queue (the tile needs ~60% of the CU's
     // 64 B/clk vector-memory path).
-    auto issue_piece = [&](int g, int ring, int idx) {
+    auto issue_piece = [&](int g, int ring, int idx) __attribute__((always_inline)) {
         uint32_t* stage = lds + ring * L::kStageDwords;
         if (idx < kXOps) {
             uint32_t* xbuf = stage + (kXOps * 4 * w) * 64;  // this wave's X rows
-            __builtin_amdgcn_global_load_lds((gptr_t)(xsrc[idx] + 128 * g), (lptr_t)(xbuf + idx * 256), 16, 0, 0);
+            const char* xg = reinterpret_cast<const char*>(a.X + 128 * g);  // uniform
+            __builtin_amdgcn_global_load_lds((gptr_t)(xg + xsrc[idx]), (lptr_t)(xbuf + idx * 256), 16, 0, 0);
         } else if (idx < kXOps + 2) {
             uint32_t* bbuf = stage + L::kXDwords + w * 512 + (idx - kXOps) * 256;
-            const u32x4* rowp = strip_w + (size_t)(8 * g + 4 * (idx - kXOps)) * N4;
-            __builtin_amdgcn_global_load_lds((gptr_t)rowp, (lptr_t)bbuf, 16, 0, 0);
+            const u32x4* rowp = strip_w + (size_t)(8 * g + 4 * (idx - kXOps)) * N4;  // uniform
+            __builtin_amdgcn_global_load_lds((gptr_t)(rowp + piece_off), (lptr_t)bbuf, 16, 0, 0);
         } else {
             // scales of the group (row 0 in per-column mode, unused then)
             uint32_t* sbuf = stage + L::kXDwords + L::kBDwords + w * 64;
             const half_t* ssrc = strip_s + (a.per_column ? (size_t)0 : (size_t)g * a.N);
-            if (dkq == 0) __builtin_amdgcn_global_load_lds((gptr_t)ssrc, (lptr_t)sbuf, 16, 0, 0);
+            if (dkq == 0) __builtin_amdgcn_global_load_lds((gptr_t)(ssrc + 8 * dslot), (lptr_t)sbuf, 16, 0, 0);
         }
     };
-    auto issue_stage = [&](int g, int ring) {
+    auto issue_stage = [&](int g, int ring) __attribute__((always_inline)) {
 #pragma unroll
         for (int idx = 0; idx < kStageOps; ++idx) issue_piece(g, ring, idx);
     };
@@ -188,111 +190,190 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     const int boff = (c8 + 8 * ch + 32 * h) * 4 + 2 * jl;  // piece kq = 2h, words 2jl, 2jl+1; kq = 2h+1 is 64 dwords on
     const int soff = (8 * ch + c8) * 4 + 2 * jl;
 
-    // next_g >= 0: also issue the loads of group next_g into slot next_ring, between the MFMA blocks
-    auto compute_stage = [&](int ring, int next_g, int next_ring) {
+    // Operands in registers.  pw[set][t][0/1]: the packed words (pieces kq = 2h, 2h+1) of packed
+    // row w + 4t; scv[set]: the lane's four scales; two sets because the next stage's words are
+    // read while the current ones are still being expanded.  xa0 / xa1: A operands of the two
+    // packed rows for every M tile (one set each: xa0 is dead after the first half of a stage
+    // and is refilled for the next stage during the second half).
+    u32x2 pw[2][2][2];   // set 0: stage being multiplied, set 1: the next one (copied over at the end)
+    u32x2 scv[2];
+    h8 xa0[MT], xa1[MT];
+    auto read_words = [&](int set, int ring) __attribute__((always_inline)) {
         const uint32_t* stage = lds + ring * L::kStageDwords;
         const uint32_t* bbuf = stage + L::kXDwords + w * 512;
-        u32x2 sc_cur = sc_fixed;
-        if (!a.per_column)
-            sc_cur = *reinterpret_cast<const u32x2*>(stage + L::kXDwords + L::kBDwords + w * 64 + soff);
+        const u32x2 sc_lds = *reinterpret_cast<const u32x2*>(stage + L::kXDwords + L::kBDwords + w * 64 + soff);
+        scv[set] = a.per_column ? sc_fixed : sc_lds;
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
-            const u32x2 p0 = *reinterpret_cast<const u32x2*>(bbuf + t * 256 + boff);
-            const u32x2 p1 = *reinterpret_cast<const u32x2*>(bbuf + t * 256 + boff + 64);
-            h8 xa[MT];
+            pw[set][t][0] = *reinterpret_cast<const u32x2*>(bbuf + t * 256 + boff);
+            pw[set][t][1] = *reinterpret_cast<const u32x2*>(bbuf + t * 256 + boff + 64);
+        }
+    };
+    auto read_xa = [&](h8 (&xa)[MT], int ring, int t) __attribute__((always_inline)) {
+        const uint32_t* stage = lds + ring * L::kStageDwords;
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const u32x2 lo = *reinterpret_cast<const u32x2*>(stage + mt * 2048 + xoff[t][0]);
-                const u32x2 hi = *reinterpret_cast<const u32x2*>(stage + mt * 2048 + xoff[t][1]);
-                const h2 d0 = bits_to_h2(lo.x), d1 = bits_to_h2(lo.y), d2 = bits_to_h2(hi.x), d3 = bits_to_h2(hi.y);
-                xa[mt] = h8{d0.x, d0.y, d1.x, d1.y, d2.x, d2.y, d3.x, d3.y};
+        for (int mt = 0; mt < MT; ++mt) {
+            const u32x2 lo = *reinterpret_cast<const u32x2*>(stage + mt * 2048 + xoff[t][0]);
+            const u32x2 hi = *reinterpret_cast<const u32x2*>(stage + mt * 2048 + xoff[t][1]);
+            const h2 d0 = bits_to_h2(lo.x), d1 = bits_to_h2(lo.y), d2 = bits_to_h2(hi.x), d3 = bits_to_h2(hi.y);
+            xa[mt] = h8{d0.x, d0.y, d1.x, d1.y, d2.x, d2.y, d3.x, d3.y};
+        }
+    };
+    auto expand = [&](int set, int block) __attribute__((always_inline)) -> h8 {  // block = 4 t + 2 jo + blk
+        const int t = block >> 2, jo = (block >> 1) & 1, blk = block & 1;
+        const h2 pr = bits_to_h2(scv[set][jo]);
+        const uint32_t q0 = blk ? (pw[set][t][0][jo] >> 8) : pw[set][t][0][jo];
+        const uint32_t q1 = blk ? (pw[set][t][1][jo] >> 8) : pw[set][t][1][jo];
+        const h2 sv = blk ? h2{pr.y, pr.y} : h2{pr.x, pr.x};
+        // K order of the operand: 4h, 4h+1 | 4h+2, 4h+3 | 4h+8, 4h+9 | 4h+10, 4h+11
+        const h2 e0 = magic.pair_low(q0) * sv, e1 = magic.pair_low(q1) * sv;
+        const h2 e2 = magic.pair_high(q0) * sv, e3 = magic.pair_high(q1) * sv;
+        return h8{e0.x, e0.y, e1.x, e1.y, e2.x, e2.y, e3.x, e3.y};
+    };
+    // Four of the eight blocks of a stage (2 packed rows x 4 B operands, MT MFMAs each).  The
+    // expansion of the following block is written between the MFMAs of a block, and so are
+    // the LDS-DMA loads of group next_g (first half only); the scheduler is told to keep that
+    // interleaving, because with one wave per SIMD nothing else fills the matrix pipe's shadow.
+    auto half_stage = [&](int set, int t, h8 (&xa)[MT], h8& bw, bool with_dma, int next_g, int next_ring) __attribute__((always_inline)) {
+#pragma unroll
+        for (int op = 0; op < 4; ++op) {
+            const int block = 4 * t + op;
+            const h8 bw_next = block < 7 ? expand(set, block + 1) : expand(set ^ 1, 0);
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt)
+                acc[mt][op] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xa[mt], bw, acc[mt][op], 0, 0, 0);
+            if (with_dma) {
+#pragma unroll
+                for (int idx = op; idx < kStageOps; idx += 4) issue_piece(next_g, next_ring, idx);
             }
+            bw = bw_next;
+        }
 #pragma unroll
-            for (int jo = 0; jo < 2; ++jo) {
-                const h2 pr = bits_to_h2(sc_cur[jo]);
-#pragma unroll
-                for (int blk = 0; blk < 2; ++blk) {
-                    const uint32_t q0 = blk ? (p0[jo] >> 8) : p0[jo];
-                    const uint32_t q1 = blk ? (p1[jo] >> 8) : p1[jo];
-                    const h2 sv = blk ? h2{pr.y, pr.y} : h2{pr.x, pr.x};
-                    // K order of the operand: 4h, 4h+1 | 4h+2, 4h+3 | 4h+8, 4h+9 | 4h+10, 4h+11
-                    const h2 e0 = magic.pair_low(q0) * sv, e1 = magic.pair_low(q1) * sv;
-                    const h2 e2 = magic.pair_high(q0) * sv, e3 = magic.pair_high(q1) * sv;
-                    const h8 bw = h8{e0.x, e0.y, e1.x, e1.y, e2.x, e2.y, e3.x, e3.y};
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-                        acc[mt][2 * jo + blk] =
-                            __builtin_amdgcn_mfma_f32_32x32x16_f16(xa[mt], bw, acc[mt][2 * jo + blk], 0, 0, 0);
-                    if (next_g >= 0) {  // uniform
-                        const int block = 4 * t + 2 * jo + blk;  // 0..7
-#pragma unroll
-                        for (int idx = block; idx < kStageOps; idx += 8) issue_piece(next_g, next_ring, idx);
-                    }
-                }
-            }
+        for (int i = 0; i < 4 * MT; ++i) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // 1 MFMA
+            __builtin_amdgcn_sched_group_barrier(0x002, MT == 4 ? 4 : (MT == 2 ? 8 : 16), 0);  // VALU
+            if (with_dma && i % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // 1 VMEM read
         }
     };
 
     // ---- software pipeline over the K groups ----------------------------------------------
-    if (ngroups > 0) issue_stage(g_begin, 0);
-    if (ngroups > 1) issue_stage(g_begin + 1, 1);
-    int ring = 0;
-    for (int it = 0; it < ngroups; ++it) {
-        // stage it+1 may stay in flight; stage it has landed once only that one is outstanding
-        if (it + 1 < ngroups) UNIQL_WAIT_VMCNT(kStageOps);
-        else UNIQL_WAIT_VMCNT(0);
-        __builtin_amdgcn_s_barrier();  // all waves' parts of stage `it` are in LDS, and everyone has
-                                       // finished reading the slot that is refilled next
-        const int refill = ring == 0 ? kRing - 1 : ring - 1;  // == (it + 2) % kRing
-        compute_stage(ring, it + 2 < ngroups ? g_begin + it + 2 : -1, refill);
-        ring = ring + 1 == kRing ? 0 : ring + 1;
+    // Iteration `it` multiplies stage `it`.  First half: packed row w (A operands xa0), while
+    // the LDS-DMA loads of stage it+2 are issued and the A operands of packed row w+4 are
+    // read from LDS.  Middle: the wave waits for stage it+1 (only the loads just issued may
+    // remain outstanding) and the workgroup meets at a barrier.  Second half: packed row w+4
+    // (xa1), while the words, scales and first-row A operands of stage it+1 are read from LDS.
+    // So the matrix pipe never waits for the barrier or for LDS.  The barrier also guarantees
+    // that every wave has finished reading the ring slot that the next iteration's loads
+    // overwrite.  Past the end the "next" group is the last one again (loaded into a slot
+    // nobody reads): no branches in the loop body and constant vmcnt arithmetic.
+    const int g_last = g_end - 1;
+    h8 bw;
+    if (ngroups > 0) {
+        issue_stage(g_begin, 0);
+        issue_stage(ngroups > 1 ? g_begin + 1 : g_last, 1);
+        UNIQL_WAIT_VMCNT(kStageOps);
+        __builtin_amdgcn_s_barrier();
+        read_words(0, 0);
+        read_xa(xa0, 0, 0);
+        bw = expand(0, 0);
     }
+    int slot = 0;
+    for (int it = 0; it < ngroups; ++it) {
+        const int slot_next = slot + 1 == kRing ? 0 : slot + 1;
+        const int slot_refill = slot_next + 1 == kRing ? 0 : slot_next + 1;
+        const int next_g = g_begin + it + 2 < g_end ? g_begin + it + 2 : g_last;
+        read_xa(xa1, slot, 1);
+        half_stage(0, 0, xa0, bw, true, next_g, slot_refill);
+        UNIQL_WAIT_VMCNT(kStageOps);   // stage it+1 has landed; only stage it+2's loads are outstanding
+        __builtin_amdgcn_s_barrier();
+        read_words(1, slot_next);
+        read_xa(xa0, slot_next, 0);
+        half_stage(0, 1, xa1, bw, false, 0, 0);
+#pragma unroll
+        for (int t = 0; t < 2; ++t) {
+            pw[0][t][0] = pw[1][t][0];
+            pw[0][t][1] = pw[1][t][1];
+        }
+        scv[0] = scv[1];
+        slot = slot_next;
+    }
+    UNIQL_WAIT_VMCNT(0);
     __syncthreads();
 
     // ---- add the four waves' partial tiles, one 32-row M tile at a time ---------------------
     // acc[mt][2 jo + blk][v] on lane l: row 32 mt + 8 (v / 4) + 4 h + v % 4,
-    // column 64 ch + 16 (2 jl + jo) + 8 blk + c8 of the strip.
-    float* red = reinterpret_cast<float*>(lds);  // [4 waves][32 rows][128 columns]
-    const int col_out = tid & 127;
-    const int n_out = 128 * strip + col_out;
+    // column 64 ch + 16 (2 jl + jo) + 8 blk + c8 of the strip.  Every wave writes its partial
+    // tile to LDS (row stride 132 floats: rows 4 apart fall on different banks); then each
+    // thread adds the four partials of two (row, 8 consecutive columns) units and stores
+    // each unit with one 16-byte store.
+    constexpr int kRedStride = 132;
+    float* red = reinterpret_cast<float*>(lds);  // [4 waves][32 rows][132]
+    const bool split_k = a.splits > 1;
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         if (m0 + mt * 32 < a.M) {  // uniform
             if (mt > 0) __syncthreads();
+            {
+                float* wred = red + w * 32 * kRedStride + (4 * h) * kRedStride + 64 * ch + 32 * jl + c8;
 #pragma unroll
-            for (int op = 0; op < 4; ++op) {
-                const int ncol = 64 * ch + 16 * (2 * jl + (op >> 1)) + 8 * (op & 1) + c8;
+                for (int op = 0; op < 4; ++op)
 #pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    red[(w * 32 + 8 * (v >> 2) + 4 * h + (v & 3)) * 128 + ncol] = acc[mt][op][v];
+                    for (int v = 0; v < 16; ++v)
+                        wred[(8 * (v >> 2) + (v & 3)) * kRedStride + 16 * (op >> 1) + 8 * (op & 1)] = acc[mt][op][v];
             }
             __syncthreads();
+            if (!split_k) {
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                const int ml = (tid >> 7) + 2 * i;
-                const int m = m0 + mt * 32 + ml;
-                if (m < a.M) {
-                    const float sum = (red[(0 * 32 + ml) * 128 + col_out] + red[(1 * 32 + ml) * 128 + col_out]) +
-                                      (red[(2 * 32 + ml) * 128 + col_out] + red[(3 * 32 + ml) * 128 + col_out]);
-                    float outv = sum;
-                    bool emit = true;
-                    unsigned long long* slot_ptr = nullptr;
-                    if (a.splits > 1) {
+                for (int u2 = 0; u2 < 2; ++u2) {
+                    const int unit = tid + 256 * u2;
+                    const int row = unit >> 4, c0 = (unit & 15) * 8;
+                    const int m = m0 + mt * 32 + row;
+                    const float* src = red + row * kRedStride + c0;
+                    f4 lo = *reinterpret_cast<const f4*>(src), hi = *reinterpret_cast<const f4*>(src + 4);
+#pragma unroll
+                    for (int ww = 1; ww < 4; ++ww) {
+                        lo += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride);
+                        hi += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride + 4);
+                    }
+                    if (m < a.M) {
+                        const size_t o = (size_t)m * a.N + 128 * strip + c0;
+                        if (a.out_f32) {
+                            float* d = reinterpret_cast<float*>(a.D) + o;
+                            *reinterpret_cast<f4*>(d) = lo;
+                            *reinterpret_cast<f4*>(d + 4) = hi;
+                        } else {
+                            const h2 r0 = h2{(half_t)lo[0], (half_t)lo[1]}, r1 = h2{(half_t)lo[2], (half_t)lo[3]};
+                            const h2 r2 = h2{(half_t)hi[0], (half_t)hi[1]}, r3 = h2{(half_t)hi[2], (half_t)hi[3]};
+                            *reinterpret_cast<u32x4*>(reinterpret_cast<half_t*>(a.D) + o) =
+                                u32x4{h2_to_bits(r0), h2_to_bits(r1), h2_to_bits(r2), h2_to_bits(r3)};
+                        }
+                    }
+                }
+            } else {
+                // K is also split over workgroups: one atomic per element, neighbouring lanes on
+                // neighbouring words (a wave touches 512 contiguous bytes per instruction)
+                const int col_out = tid & 127;
+                for (int i = 0; i < 16; ++i) {
+                    const int row = (tid >> 7) + 2 * i;
+                    const int m = m0 + mt * 32 + row;
+                    if (m < a.M) {
+                        const float* src = red + row * kRedStride + col_out;
+                        const float sum = (src[0] + src[32 * kRedStride]) + (src[64 * kRedStride] + src[96 * kRedStride]);
+                        const size_t o = (size_t)m * a.N + 128 * strip + col_out;
                         const float v = fminf(fmaxf(sum, -kTileAccumClamp), kTileAccumClamp);
                         const long long fixed = __float2ll_rn(v * kTileAccumScale);
                         const unsigned long long word = ((unsigned long long)fixed << 8) + 1ull;
-                        slot_ptr = a.accum + (size_t)m * a.N + n_out;
+                        unsigned long long* slot_ptr = a.accum + o;
                         const unsigned long long old =
                             __hip_atomic_fetch_add(slot_ptr, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        emit = ((int)(old & 0xffull) == a.splits - 1);
-                        outv = (float)((long long)(old + word) >> 8) * (1.0f / kTileAccumScale);
-                    }
-                    if (emit) {
-                        if (a.out_f32)
-                            reinterpret_cast<float*>(a.D)[(size_t)m * a.N + n_out] = outv;
-                        else
-                            reinterpret_cast<half_t*>(a.D)[(size_t)m * a.N + n_out] = (half_t)outv;
-                        if (slot_ptr) __hip_atomic_store(slot_ptr, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        if ((int)(old & 0xffull) == a.splits - 1) {
+                            const float outv = (float)((long long)(old + word) >> 8) * (1.0f / kTileAccumScale);
+                            if (a.out_f32)
+                                reinterpret_cast<float*>(a.D)[o] = outv;
+                            else
+                                reinterpret_cast<half_t*>(a.D)[o] = (half_t)outv;
+                            __hip_atomic_store(slot_ptr, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        }
                     }
                 }
             }
@@ -306,16 +387,17 @@ static inline int ceil_div_i(int a, int b) { return (a + b - 1) / b; }
 struct TilePlan {
     int mtiles, splits, gps;
 };
-static TilePlan tile_plan(int m, int n, int k, int splits_override);
+static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_override = 0);
 
 size_t tile_accum_bytes(int m, int n, int k) {
     // one word per output element, only when the plan splits K over workgroups
     return tile_plan(m, n, k, 0).splits > 1 ? (size_t)m * n * sizeof(unsigned long long) : 0;
 }
 
-static TilePlan tile_plan(int m, int n, int k, int splits_override) {
+static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_override) {
     TilePlan p;
     p.mtiles = m <= 32 ? 1 : (m <= 64 ? 2 : 4);  // 32-row M tiles per workgroup
+    if (mt_override == 1 || mt_override == 2 || mt_override == 4) p.mtiles = mt_override;
     const int G = k / 128;
     const int tiles = (n / 128) * ceil_div_i(m, 32 * p.mtiles);
     int splits = 1;
@@ -345,10 +427,11 @@ static hipError_t tile_launch_one(const TileArgs& a, int grid, hipStream_t strea
     return hipGetLastError();
 }
 
-// tune: bits 0..7 force the number of K splits (0 = choose)
+// tune: bits 0..7 force the number of K splits, bits 8..11 the number of 32-row M tiles per
+// workgroup (0 = choose)
 int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, void* accum, size_t accum_bytes,
                 int m, int n, int k, int groups, bool out_f32, unsigned tune, hipStream_t stream) {
-    const TilePlan plan = tile_plan(m, n, k, (int)(tune & 0xffu));
+    const TilePlan plan = tile_plan(m, n, k, (int)(tune & 0xffu), (int)((tune >> 8) & 0xfu));
     if (plan.splits > 1 && (!accum || accum_bytes < (size_t)m * n * sizeof(unsigned long long)))
         return UNIQL_E_WORKSPACE;
     TileArgs a;
