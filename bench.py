@@ -37,6 +37,10 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 LLC_BYTES = 256 << 20
+# HBM bytes per launch of the default workload (mean over the four linears) from two
+# rocprofv3 --pmc runs of this file, FETCH_SIZE and WRITE_SIZE, each scaled by the reading for a
+# 128 MiB elementwise copy (--pmc-calibrate): factors 2.000 and 1.000.
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28838246
 
 LLAMA_DECODE = [("qkv", 4096, 6144), ("o_proj", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
 PRUNED = [("q_pruned", 4096, 3584, 0), ("o_pruned", 3456, 4096, 0), ("gate_up_pruned", 4096, 24320, 0),
@@ -224,6 +228,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--pmc-calibrate", action="store_true",
+                    help="also launch three plain elementwise copies of 128 MiB (read 128 MiB, write 128 MiB each) "
+                         "before the timed region: the known-size kernel a rocprofv3 --pmc run scales its "
+                         "FETCH_SIZE / WRITE_SIZE readings by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: this path has no multi-GPU leg (run with --gpus 1)", file=sys.stderr)
@@ -236,6 +244,14 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     gen = torch.Generator(device=dev).manual_seed(1234)
+
+    if args.pmc_calibrate:
+        src = torch.ones(64 << 20, dtype=torch.float16, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            torch.mul(src, 1.0, out=dst)
+        torch.cuda.synchronize()
+        del src, dst
 
     m = 1
     step_bytes = sum(linear_bytes(m, k, n) for _, k, n in LLAMA_DECODE)
@@ -259,8 +275,8 @@ def main():
                    "m": m, "group_size": 128, "weight_copies_rotated": copies, "launch": "hip_graph",
                    "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "wall_ms_per_step": round(wall_per_step * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None,
-                     "kernel": "w4a16_stream_kernel<1,false>", "launches_per_step": launches,
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
+                     "kernel": "w4a16_stream_kernel<MT=1,HAD=false> (all four launches of a step)", "launches_per_step": launches,
                      "avg_launch_us": round(kernel_us, 3), "bytes_per_launch": step_bytes // launches},
     }
     del layers
