@@ -33,6 +33,31 @@ def reference_product(p, exact=False):
     return O.gemm_fp64(p["x"], w) if exact else O.gemm_fp32(p["x"], w)
 
 
+def unrounded_product(p, x=None):
+    """x . ((q - 8) s) in float64 with the weights NOT rounded to fp16: what the streaming
+    kernel computes (scale applied to each group's fp32 dot product) up to fp32 rounding."""
+    k, n = p["k"], p["n"]
+    group = k if p["s"].shape[0] == 1 else 128
+    s_full = np.repeat(p["s"].astype(np.float64), group, axis=0)
+    w = (p["q"].astype(np.float64) - 8.0) * s_full
+    return (p["x"] if x is None else x).astype(np.float64) @ w
+
+
+def check_fp32_result(y32, p, ref, m, x=None, forced_stream=False):
+    """fp32 output against the float64 product.  The tiled kernel (m > 16) multiplies the
+    reference's fp16-rounded weights: only fp32 accumulation error remains.  The streaming
+    kernel (m <= 16) scales each group's dot product of raw codes: the same holds against the
+    product with unrounded weights, and the distance to `ref` is the weights' rounding noise."""
+    if m <= 16 or forced_stream:
+        d = np.abs(y32 - unrounded_product(p, x)).max()
+        assert d < 2e-4, d
+        d = np.abs(y32 - ref).max()
+        assert d < 1e-4 * np.sqrt(p["k"]), d   # ~ 2^-11 relative noise per weight, summed over K
+    else:
+        d = np.abs(y32 - ref).max()
+        assert d < 2e-4, d
+
+
 def fp16_half_ulp(ref):
     """Half the fp16 spacing at |ref| (normal range)."""
     a = np.maximum(np.abs(ref).astype(np.float64), 2.0 ** -14)
@@ -42,13 +67,15 @@ def fp16_half_ulp(ref):
 def check_layer_output(y16, ref, *, max_abs=1e-2, mean_rel=1e-3):
     """The path's tolerance: max-abs 1e-2 and mean relative 1e-3 against the
     fp32-accumulated reference.  An fp16 result cannot be closer to the reference than
-    half an fp16 ulp of it (0.0156 once |y| >= 32), so the absolute bound is
-    max(1e-2, half ulp + 1e-3): the first term is the stated tolerance, the second the
-    representation floor."""
+    half an fp16 ulp of it (0.0078 once |y| >= 16, 0.0156 once |y| >= 32), so the absolute
+    bound is max(1e-2, half ulp + 5e-3): the first term is the stated tolerance, the second
+    the representation floor plus half the tolerance for the value before rounding (the
+    streaming kernel does not round the scaled weights to fp16 as the reference does, which
+    moves that value by up to about 4e-3 at K = 14336)."""
     y = np.asarray(y16, dtype=np.float64)
     ref = np.asarray(ref, dtype=np.float64)
     err = np.abs(y - ref)
-    bound = np.maximum(max_abs, fp16_half_ulp(ref) + 1e-3)
+    bound = np.maximum(max_abs, fp16_half_ulp(ref) + 0.5 * max_abs)
     assert (err <= bound).all(), f"max abs err {err.max():.4g} at |ref| {np.abs(ref).flat[err.argmax()]:.3g}"
     rel = err.sum() / np.abs(ref).sum()
     assert rel <= mean_rel, f"mean relative error {rel:.3g}"

@@ -5,7 +5,7 @@ import torch
 
 from oracle import uniql_oracle as O
 from tests.helpers import (check_layer_output, make_linear_problem, reference_product, to_gpu,
-                           workspace_for)
+                           check_fp32_result, workspace_for)
 
 pytestmark = pytest.mark.gpu
 
@@ -67,7 +67,7 @@ def test_stream_kernel_small_m(gpu, m, k, n):
     p = make_linear_problem(m, k, n, seed=100 * m + k // 128 + n)
     ref = reference_product(p, exact=True)
     y32 = run_gemm(p, gpu, out_f32=True)
-    assert np.abs(y32 - ref).max() < 2e-4, np.abs(y32 - ref).max()     # fp32 accumulation only
+    check_fp32_result(y32, p, ref, m)
     y16 = run_gemm(p, gpu)
     assert np.array_equal(y16.view(np.uint16), y32.astype(np.float16).view(np.uint16))
     check_layer_output(y16, ref)
@@ -91,7 +91,7 @@ def test_stream_kernel_forced_for_larger_m(gpu, m):
     p = make_linear_problem(m, 512, 256, seed=m)
     ref = reference_product(p, exact=True)
     y32 = run_gemm(p, gpu, out_f32=True, flags=F_FORCE_SKINNY)
-    assert np.abs(y32 - ref).max() < 2e-4
+    check_fp32_result(y32, p, ref, m, forced_stream=True)
     check_layer_output(run_gemm(p, gpu, flags=F_FORCE_SKINNY), ref)
 
 
@@ -152,7 +152,7 @@ def test_units_per_wave_override(gpu, upw):
     p = make_linear_problem(2, 1408, 256, seed=upw)     # 11 groups: ragged against 4*upw
     ref = reference_product(p, exact=True)
     y32 = run_gemm(p, gpu, out_f32=True, flags=upw << 8)
-    assert np.abs(y32 - ref).max() < 2e-4
+    check_fp32_result(y32, p, ref, 2)
 
 
 def test_per_column_scales(gpu):
@@ -160,7 +160,7 @@ def test_per_column_scales(gpu):
         p = make_linear_problem(3, k, 256, seed=k, per_column=True)
         ref = reference_product(p, exact=True)
         y32 = run_gemm(p, gpu, out_f32=True)
-        assert np.abs(y32 - ref).max() < 2e-4
+        check_fp32_result(y32, p, ref, 3)
 
 
 def test_deterministic_and_repeatable(gpu):
@@ -190,7 +190,7 @@ def test_fused_blockwise_hadamard(gpu, m):
     w = O.dequant_codes(p["q"], p["s"])
     ref = O.gemm_fp64(xr, w)
     y32 = run_gemm(p, gpu, out_f32=True, had_block=128, had_scale=128 ** -0.5)
-    assert np.abs(y32 - ref).max() < 2e-4
+    check_fp32_result(y32, p, ref, m, x=xr)
     check_layer_output(run_gemm(p, gpu, had_block=128, had_scale=128 ** -0.5), ref)
 
 
@@ -201,7 +201,7 @@ def test_full_width_hadamard_prologue(gpu, m):
     xr = O.fwht(p["x"], k ** -0.5)
     ref = O.gemm_fp64(xr, O.dequant_codes(p["q"], p["s"]))
     y32 = run_gemm(p, gpu, out_f32=True, had_block=k, had_scale=k ** -0.5)
-    assert np.abs(y32 - ref).max() < 2e-4
+    check_fp32_result(y32, p, ref, m, x=xr)
 
 
 # ------------------------------------------------------------------ error paths

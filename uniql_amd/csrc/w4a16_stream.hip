@@ -9,12 +9,26 @@
 //     lane l :  slot = l % 16  ->  chunk = 2*strip + slot/8,  c8 = slot % 8
 //               kq   = l / 16  ->  piece 4*c8 + kq
 //
-// Every byte of the 1 KiB row segment is fetched once, the codes are expanded to
-// fp16 (code-8)*scale in registers exactly as the reference does, and eight MFMAs
-// (one per jb) consume two packed rows (32 K values) at a time.  The activations
-// are the A operand: rows of X (up to 16 per M-tile) staged through LDS in the same
-// K order.  MFMA is used purely as a wide dot-product unit: its cost does not
-// depend on M, so M = 1..16 all run at the weight-streaming rate.
+// Every byte of the 1 KiB row segment is fetched once and eight MFMAs (one per jb)
+// consume two packed rows (32 K values) at a time.  The activations are the A operand:
+// rows of X (up to 16 per M-tile) staged through LDS in the same K order.  MFMA is
+// used purely as a wide dot-product unit: its cost does not depend on M, so
+// M = 1..16 all run at the weight-streaming rate.
+//
+// Expanding codes to scaled fp16 weights costs 13 vector instructions per packed
+// word, which at M <= 16 is more vector work than the memory system leaves time for.
+// This kernel feeds the RAW codes to the matrix unit instead:
+//   * `word & 0x000f000f` read as two fp16 values is (code * 2^-24) twice: a
+//     subnormal, which the MFMA unit multiplies exactly.  `word & 0x00f000f0` is
+//     (16 code * 2^-24); the matching activations are staged pre-divided by 16.
+//     Five instructions per packed word (one shift, four ANDs).
+//   * the zero point: sum_k x_k (code_k - 8) = sum_k x_k code_k - 8 sum_k x_k.  The
+//     second term only depends on the activation row and the group; it is computed
+//     once while staging and enters the group's first MFMA as its C operand.
+//   * the scale multiplies the group's fp32 dot product (one FMA per output and
+//     group) instead of every weight.
+// The result is sum_g s_g . sum_k x_k (code_k - 8) with fp32 arithmetic throughout:
+// the same value as the reference's up to its fp16 rounding of every scaled weight.
 //
 // Work split: unit = (strip of 128 columns) x (group of 128 K).  A wave owns `upw`
 // consecutive groups of a strip, the four waves of a workgroup own consecutive
@@ -57,14 +71,19 @@ __device__ __forceinline__ void store_out(const StreamArgs& a, int m, int n, flo
         reinterpret_cast<half_t*>(a.D)[(size_t)m * a.N + n] = (half_t)v;
 }
 
-// MT: 16-row tiles of M per workgroup.  WAVES: wavefronts per workgroup (4, 8 or 16);
-// with 16 a workgroup can cover all of K for shapes with many strips, which removes the
-// exchange of partial sums between workgroups.  PF: prefetch the next group's weights
-// into a second register set while the current one is consumed.
-template <int MT, bool HAD, int WAVES, bool PF>
+// MT: 16-row tiles of M per workgroup.  RC: row class, an upper bound of M for MT = 1
+// (1, 2, 4, 8, 16): it fixes NV, how many of the four output rows of a lane's accumulator
+// quad are real, and XQ, how many quads of activation rows are loaded and staged.  WAVES: wavefronts
+// per workgroup (4, 8 or 16); with 16 a workgroup can cover all of K for shapes with many
+// strips, which removes the exchange of partial sums between workgroups.  PF: prefetch the
+// next group's weights into a second register set while the current one is consumed.
+template <int MT, int RC, bool HAD, int WAVES, bool PF>
 __global__ __launch_bounds__(64 * WAVES, (MT == 1 ? (WAVES == 16 ? 4 : 3) : (MT == 2 ? 2 : 1)))
 void w4a16_stream_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    constexpr int NV = RC < 4 ? RC : 4;
+    constexpr int XQ = MT > 1 ? 4 : (RC + 3) / 4;
+    constexpr int RPW = 4;  // row pairs (32 K values each) per group
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -87,35 +106,44 @@ void w4a16_stream_kernel(const StreamArgs a) {
     const u32x4* strip_w = a.B + (size_t)strip * 64;
     const half_t* strip_s = a.S + (size_t)strip * 128;
 
-    NibbleMagic magic;
-    magic.init();
-
-    f4 acc[MT][8];
+    float acc[MT][8][NV];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int jb = 0; jb < 8; ++jb) acc[mt][jb] = f4{0.f, 0.f, 0.f, 0.f};
+        for (int jb = 0; jb < 8; ++jb)
+#pragma unroll
+            for (int v = 0; v < NV; ++v) acc[mt][jb][v] = 0.f;
 
     uint32_t* xs = lds + (size_t)w * a.xrows * kXsStride;  // this wave's staging rows
+    // Staged row layout (dwords): the pair of K values 2d, 2d+1 of the group, d = 16 rp + kq' + 4 t,
+    // sits at dword 16 rp + 4 kq' + t, so that the A operand of lane (row, kq') for row pair rp
+    // is one 16-byte read; pairs with odd t (K rows 8..15 of a packed row) are stored divided
+    // by 16.  Dword 64 of the row holds 8 * 2^-24 * (sum of the row's values) as fp32.
     // MFMA row `slot` of tile mt reads staged row min(16 mt + slot, xrows - 1): rows past M
-    // only feed output rows that are never stored
+    // only feed output rows that are never stored.
     int xrow_of[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         const int r = mt * 16 + slot;
-        xrow_of[mt] = (r < a.xrows ? r : a.xrows - 1) * kXsStride + kq;
+        xrow_of[mt] = (r < a.xrows ? r : a.xrows - 1) * kXsStride + 4 * kq;
     }
+    // where this lane's staged quad goes: lane `slot` holds pairs d = 4 slot + i
+    const int stage_off = 16 * (slot >> 2) + (slot & 3);
+    const half_t stage_mul = (slot & 1) ? (half_t)0.0625f : (half_t)1.0f;
+    const h2 stage_mul2 = h2{stage_mul, stage_mul};
+    uint32_t mask_low = 0x000f000fu, mask_high = 0x00f000f0u;
+    asm volatile("" : "+s"(mask_low), "+s"(mask_high));  // keep both masks in scalar registers
 
-    u32x4 wq[8];
+    u32x4 wq[2 * RPW];
     u32x4 sc;
-    u32x4 xv[MT][4];
+    u32x4 xv[MT][XQ];
     // everything group g needs from memory: activations first (small, they gate the LDS
     // staging), then scales, then the eight packed rows
     auto issue_loads = [&](int g) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+            for (int i = 0; i < XQ; ++i) {
                 const int m = mt * 16 + i * 4 + kq;
                 xv[mt][i] = u32x4{0u, 0u, 0u, 0u};
                 if (m < a.M)
@@ -137,7 +165,7 @@ void w4a16_stream_kernel(const StreamArgs a) {
         }
         const u32x4* rowp = strip_w + (size_t)(8 * g) * N4;  // uniform
 #pragma unroll
-        for (int rr = 0; rr < 8; ++rr) wq[rr] = __builtin_nontemporal_load(rowp + (size_t)rr * N4 + piece_off);
+        for (int rr = 0; rr < 2 * RPW; ++rr) wq[rr] = __builtin_nontemporal_load(rowp + (size_t)rr * N4 + piece_off);
     };
 
     if (PF && g_begin < g_end) issue_loads(g_begin);
@@ -148,7 +176,7 @@ void w4a16_stream_kernel(const StreamArgs a) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
 #pragma unroll
-            for (int i = 0; i < 4; ++i) {
+            for (int i = 0; i < XQ; ++i) {
                 const int mrow = mt * 16 + i * 4;
                 if (mrow < a.xrows) {  // uniform
                     u32x4 v = xv[mt][i];
@@ -169,7 +197,19 @@ void w4a16_stream_kernel(const StreamArgs a) {
                             v[p] = h2_to_bits(hv);
                         }
                     }
-                    *reinterpret_cast<u32x4*>(xs + (size_t)(mrow + kq) * kXsStride + 4 * slot) = v;
+                    // 8 * 2^-24 * (sum of the row), from the values the MFMA will see
+                    float sum = 0.f;
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) {
+                        const h2 hv = bits_to_h2(v[p]);
+                        sum += (float)hv.x + (float)hv.y;
+                    }
+#pragma unroll
+                    for (int d = 1; d < 16; d <<= 1) sum += __shfl_xor(sum, d, kWave);
+                    uint32_t* row = xs + (size_t)(mrow + kq) * kXsStride;
+#pragma unroll
+                    for (int p = 0; p < 4; ++p) row[stage_off + 4 * p] = h2_to_bits(bits_to_h2(v[p]) * stage_mul2);
+                    if (slot == 0) reinterpret_cast<float*>(row)[64] = sum * (8.0f / kAccumScale);
                 }
             }
         }
@@ -179,79 +219,108 @@ void w4a16_stream_kernel(const StreamArgs a) {
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        u32x4 cur[8];
+        u32x4 cur[2 * RPW];
 #pragma unroll
-        for (int rr = 0; rr < 8; ++rr) cur[rr] = wq[rr];
+        for (int rr = 0; rr < 2 * RPW; ++rr) cur[rr] = wq[rr];
         const u32x4 sc_cur = sc;
         // all activation rows this group needs, fetched from LDS before the next group's
         // loads overwrite the staging registers
-        h8 xa[4][MT];
+        h8 xa[RPW][MT];
+        f4 zp[MT];  // minus 8 * row sums for this lane's four output rows: the first MFMA's C operand
 #pragma unroll
-        for (int rp = 0; rp < 4; ++rp) {
+        for (int mt = 0; mt < MT; ++mt) {
+            if (PF || WAVES != 16) {
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                const uint32_t* xr = xs + xrow_of[mt] + 16 * rp;
-                const h2 d0 = bits_to_h2(xr[0]), d1 = bits_to_h2(xr[4]);
-                const h2 d2 = bits_to_h2(xr[8]), d3 = bits_to_h2(xr[12]);
-                xa[rp][mt] = h8{d0.x, d0.y, d1.x, d1.y, d2.x, d2.y, d3.x, d3.y};
+                for (int rp = 0; rp < RPW; ++rp)
+                    xa[rp][mt] = __builtin_bit_cast(
+                        h8, *reinterpret_cast<const u32x4*>(xs + xrow_of[mt] + 16 * rp));
+            }
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int r = mt * 16 + 4 * kq + v;
+                const float* sums = reinterpret_cast<const float*>(xs) + (r < a.xrows ? r : a.xrows - 1) * kXsStride + 64;
+                zp[mt][v] = (v >= NV) ? 0.f : -sums[0];
             }
         }
         if (PF && g + 1 < g_end) issue_loads(g + 1);
 
-        h2 s2[8];
+        // two passes over the columns (word pairs j) keep the group's raw dot products in
+        // sixteen registers; the scale of output column jb of this lane is half jb of the
+        // 16-byte scale load
 #pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            const h2 pr = bits_to_h2(sc_cur[p]);
-            s2[2 * p] = h2{pr.x, pr.x};
-            s2[2 * p + 1] = h2{pr.y, pr.y};
-        }
-
+        for (int jh = 0; jh < 2; ++jh) {
+            f4 dot[MT][4];
 #pragma unroll
-        for (int rp = 0; rp < 4; ++rp) {
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const uint32_t q0 = cur[2 * rp][j], q1 = cur[2 * rp + 1][j];
-#pragma unroll
-                for (int blk = 0; blk < 2; ++blk) {
-                    const uint32_t p0 = blk ? (q0 >> 8) : q0;
-                    const uint32_t p1 = blk ? (q1 >> 8) : q1;
-                    const h2 sv = s2[2 * j + blk];
-                    const h2 e0 = magic.pair_low(p0) * sv, e1 = magic.pair_high(p0) * sv;
-                    const h2 e2 = magic.pair_low(p1) * sv, e3 = magic.pair_high(p1) * sv;
-                    const h8 bw = h8{e0.x, e0.y, e1.x, e1.y, e2.x, e2.y, e3.x, e3.y};
+            for (int rp = 0; rp < RPW; ++rp) {
+                // 16-wave workgroups live on 128 registers: they re-read the activations from
+                // LDS in each pass instead of holding all four row pairs
+                if (!PF && WAVES == 16) {
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
-                        acc[mt][2 * j + blk] =
-                            __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[rp][mt], bw, acc[mt][2 * j + blk], 0, 0, 0);
+                        xa[rp][mt] = __builtin_bit_cast(
+                            h8, *reinterpret_cast<const u32x4*>(xs + xrow_of[mt] + 16 * rp));
                 }
+#pragma unroll
+                for (int jl = 0; jl < 2; ++jl) {
+                    const int j = 2 * jh + jl;
+                    const uint32_t q0 = cur[2 * rp][j], q1 = cur[2 * rp + 1][j];
+#pragma unroll
+                    for (int blk = 0; blk < 2; ++blk) {
+                        const uint32_t p0 = blk ? (q0 >> 8) : q0;
+                        const uint32_t p1 = blk ? (q1 >> 8) : q1;
+                        const u32x4 raw = u32x4{p0 & mask_low, p0 & mask_high, p1 & mask_low, p1 & mask_high};
+                        const h8 bw = __builtin_bit_cast(h8, raw);
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt)
+                            dot[mt][2 * jl + blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                                xa[rp][mt], bw, rp == 0 ? zp[mt] : dot[mt][2 * jl + blk], 0, 0, 0);
+                    }
+                }
+            }
+#pragma unroll
+            for (int jq = 0; jq < 4; ++jq) {
+                const int jb = 4 * jh + jq;
+                const h2 pr = bits_to_h2(sc_cur[jb >> 1]);
+                const float sf = (float)((jb & 1) ? pr.y : pr.x);
+#pragma unroll
+                for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+                    for (int v = 0; v < NV; ++v) acc[mt][jb][v] += dot[mt][jq][v] * sf;
             }
         }
     }
 
-    // ---- combine the waves (four at a time, fixed order), then the K splits -----------
+    // ---- combine the waves (fixed order), then the K splits ------------------------------
     // acc[mt][jb][v] on lane l is row m = 16 mt + 4 (l/16) + v, column
     // 128 strip + 64 (slot/8) + 16 (jb/2) + 8 (jb%2) + slot%8.
-    float* red = reinterpret_cast<float*>(lds);  // [4 waves][16 rows][128 columns]
-    constexpr int RPT = WAVES / 2;               // output rows covered per pass of the workgroup
-    constexpr int NI = 16 / RPT;                 // passes needed for 16 rows
+    // The exchange area follows the staging rows, so no barrier is needed before the first
+    // round.  With at most four activation rows all waves fit one round.
+    float* red = reinterpret_cast<float*>(lds + (size_t)WAVES * a.xrows * kXsStride);
+    const int rr_rows = a.xrows <= 4 ? 4 : 16;      // rows per wave in the exchange area
+    const int wpr = a.xrows <= 4 ? WAVES : 4;       // waves per round
+    constexpr int RPT = WAVES / 2;                  // output rows covered per pass of the workgroup
+    constexpr int NI = 16 / RPT;                    // passes needed for 16 rows
     const int ncol_lane = 64 * (slot >> 3) + c8;
     const int col_out = tid & 127;
     const int n_out = 128 * strip + col_out;
+    bool first_round = true;
     for (int mt = 0; mt < MT; ++mt) {
         if (mt * 16 >= a.M) break;
         float tot[NI];
 #pragma unroll
         for (int i = 0; i < NI; ++i) tot[i] = 0.f;
-        for (int round = 0; round < WAVES / 4; ++round) {
-            __syncthreads();
-            if ((w >> 2) == round) {
+        for (int round = 0; round < WAVES / wpr; ++round) {
+            if (!first_round) __syncthreads();
+            first_round = false;
+            if (w / wpr == round) {
 #pragma unroll
                 for (int jb = 0; jb < 8; ++jb) {
 #pragma unroll
-                    for (int v = 0; v < 4; ++v) {
+                    for (int v = 0; v < NV; ++v) {
                         const int ml = 4 * kq + v;
                         if (mt * 16 + ml < a.M)
-                            red[((w & 3) * 16 + ml) * 128 + ncol_lane + 16 * (jb >> 1) + 8 * (jb & 1)] = acc[mt][jb][v];
+                            red[((w % wpr) * rr_rows + ml) * 128 + ncol_lane + 16 * (jb >> 1) + 8 * (jb & 1)] =
+                                acc[mt][jb][v] * kAccumScale;
                     }
                 }
             }
@@ -259,9 +328,9 @@ void w4a16_stream_kernel(const StreamArgs a) {
 #pragma unroll
             for (int i = 0; i < NI; ++i) {
                 const int ml = (tid >> 7) + RPT * i;
-                if (mt * 16 + ml < a.M)
-                    tot[i] += (red[(0 * 16 + ml) * 128 + col_out] + red[(1 * 16 + ml) * 128 + col_out]) +
-                              (red[(2 * 16 + ml) * 128 + col_out] + red[(3 * 16 + ml) * 128 + col_out]);
+                if (mt * 16 + ml < a.M) {
+                    for (int ww = 0; ww < wpr; ++ww) tot[i] += red[(ww * rr_rows + ml) * 128 + col_out];
+                }
             }
         }
 #pragma unroll
@@ -297,7 +366,7 @@ static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 struct StreamPlan {
     int waves;  // 4, 8 or 16
-    int upw;
+    int upw;    // groups per wave
     int splits;
 };
 
@@ -335,12 +404,12 @@ size_t stream_accum_bytes(int m, int n, int k) {
     return (size_t)mrows * n * sizeof(unsigned long long);
 }
 
-template <int MT, bool HAD, int WAVES, bool PF>
+template <int MT, int RC, bool HAD, int WAVES, bool PF>
 static hipError_t launch_one(const StreamArgs& a, hipStream_t stream) {
     const size_t stage = (size_t)WAVES * a.xrows * kXsStride * 4;
-    const size_t red = (size_t)4 * 16 * 128 * 4;
-    const size_t shmem = stage > red ? stage : red;
-    auto kern = &w4a16_stream_kernel<MT, HAD, WAVES, PF>;
+    const size_t red = a.xrows <= 4 ? (size_t)WAVES * 4 * 128 * 4 : (size_t)4 * 16 * 128 * 4;
+    const size_t shmem = stage + red;
+    auto kern = &w4a16_stream_kernel<MT, RC, HAD, WAVES, PF>;
     if (shmem > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -351,17 +420,29 @@ static hipError_t launch_one(const StreamArgs& a, hipStream_t stream) {
     return hipGetLastError();
 }
 
-template <int MT, bool HAD>
+template <int MT, int RC, bool HAD>
 static hipError_t launch_waves(const StreamArgs& a, int waves, bool pf, hipStream_t stream) {
     if constexpr (MT == 1) {
-        if (waves == 16) return launch_one<MT, HAD, 16, false>(a, stream);  // 128-register budget: no second weight set
-        if (waves == 8) return pf ? launch_one<MT, HAD, 8, true>(a, stream) : launch_one<MT, HAD, 8, false>(a, stream);
+        if (waves == 16) return launch_one<MT, RC, HAD, 16, false>(a, stream);  // 128-register budget: no second weight set
+        if (waves == 8)
+            return pf ? launch_one<MT, RC, HAD, 8, true>(a, stream) : launch_one<MT, RC, HAD, 8, false>(a, stream);
     }
-    return pf ? launch_one<MT, HAD, 4, true>(a, stream) : launch_one<MT, HAD, 4, false>(a, stream);
+    return pf ? launch_one<MT, RC, HAD, 4, true>(a, stream) : launch_one<MT, RC, HAD, 4, false>(a, stream);
+}
+
+template <bool HAD>
+static hipError_t launch_rows(const StreamArgs& a, int mt, int waves, bool pf, hipStream_t stream) {
+    if (mt == 4) return launch_waves<4, 16, HAD>(a, waves, pf, stream);
+    if (mt == 2) return launch_waves<2, 16, HAD>(a, waves, pf, stream);
+    if (a.M == 1) return launch_waves<1, 1, HAD>(a, waves, pf, stream);
+    if (a.M == 2) return launch_waves<1, 2, HAD>(a, waves, pf, stream);
+    if (a.M <= 4) return launch_waves<1, 4, HAD>(a, waves, pf, stream);
+    if (a.M <= 8) return launch_waves<1, 8, HAD>(a, waves, pf, stream);
+    return launch_waves<1, 16, HAD>(a, waves, pf, stream);
 }
 
 // Rows are processed in slabs of at most 64; every slab re-streams the weights.
-// tune: bits 0..7 groups per wave, bits 8..11 waves per workgroup (4/8/16), bit 12 no prefetch;
+// tune: bits 0..7 groups per wave, bits 8..12 waves per workgroup (4/8/16), bit 13 no prefetch;
 // zero fields mean "choose".
 int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, void* accum, int m, int n,
                   int k, int groups, bool had128, float had_scale, bool out_f32, unsigned tune,
@@ -377,7 +458,7 @@ int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void
     a.per_column = (groups == 1) ? 1 : 0;
     a.out_f32 = out_f32 ? 1 : 0;
     a.had_scale = had_scale;
-    int waves_override = (int)((tune >> 8) & 0xfu);
+    int waves_override = (int)((tune >> 8) & 0x1fu);
     if (waves_override != 4 && waves_override != 8 && waves_override != 16) waves_override = 0;
     const size_t out_elt = out_f32 ? 4 : 2;
     for (int m0 = 0; m0 < m; m0 += 64) {
@@ -390,17 +471,9 @@ int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void
         a.xrows = mt == 1 ? ((mm + 3) / 4) * 4 : mt * 16;
         a.X = reinterpret_cast<const half_t*>(A) + (size_t)m0 * lda;
         a.D = reinterpret_cast<char*>(D) + (size_t)m0 * n * out_elt;
-        const bool pf = !(tune & 0x1000u) && plan.upw > 1 && plan.waves != 16;
-        hipError_t e;
-        if (had128) {
-            if (mt == 1) e = launch_waves<1, true>(a, plan.waves, pf, stream);
-            else if (mt == 2) e = launch_waves<2, true>(a, plan.waves, pf, stream);
-            else e = launch_waves<4, true>(a, plan.waves, pf, stream);
-        } else {
-            if (mt == 1) e = launch_waves<1, false>(a, plan.waves, pf, stream);
-            else if (mt == 2) e = launch_waves<2, false>(a, plan.waves, pf, stream);
-            else e = launch_waves<4, false>(a, plan.waves, pf, stream);
-        }
+        const bool pf = !(tune & 0x2000u) && plan.upw > 1 && plan.waves != 16;
+        const hipError_t e = had128 ? launch_rows<true>(a, mt, plan.waves, pf, stream)
+                                    : launch_rows<false>(a, mt, plan.waves, pf, stream);
         if (e != hipSuccess) return UNIQL_E_LAUNCH;
     }
     return UNIQL_OK;
