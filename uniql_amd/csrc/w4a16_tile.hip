@@ -394,18 +394,40 @@ size_t tile_accum_bytes(int m, int n, int k) {
     return tile_plan(m, n, k, 0).splits > 1 ? (size_t)m * n * sizeof(unsigned long long) : 0;
 }
 
+// Measured on MI355X (K groups of 128, one 32-row tile = "row tile"):
+//   * a workgroup of MT row tiles spends about 0.7 / 1.1 / 1.4 us per K group (MT = 1 / 2 / 4)
+//     when it has a compute unit to itself; per row tile the larger ones are the more
+//     efficient (they expand every weight once for MT row tiles), and two MT = 2 workgroups
+//     sharing a compute unit match one MT = 4 workgroup;
+//   * the exchange of partial sums costs one 64-bit atomic per output element and K split,
+//     about 150 G atomics/s for the chip.
+// So: the largest MT that still yields about one workgroup per compute unit; MT = 2 instead of
+// 4 when the MT = 4 grid would leave the last round of 256 workgroups mostly empty; K splits
+// only for MT = 1 grids that cannot fill the chip, and only while the atomics cost less than
+// the K loop they save.
 static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_override) {
     TilePlan p;
-    p.mtiles = m <= 32 ? 1 : (m <= 64 ? 2 : 4);  // 32-row M tiles per workgroup
+    const int strips = n / 128, G = k / 128;
+    const int64_t t4 = (int64_t)strips * ceil_div_i(m, 128), t2 = (int64_t)strips * ceil_div_i(m, 64);
+    if (t4 >= 256) p.mtiles = (t4 % 256 == 0 || t4 >= 1024) ? 4 : 2;
+    else if (t2 >= 200) p.mtiles = 2;
+    else p.mtiles = 1;
+    if (m <= 32) p.mtiles = 1;
     if (mt_override == 1 || mt_override == 2 || mt_override == 4) p.mtiles = mt_override;
-    const int G = k / 128;
-    const int tiles = (n / 128) * ceil_div_i(m, 32 * p.mtiles);
+    const int64_t tiles = (int64_t)strips * ceil_div_i(m, 32 * p.mtiles);
     int splits = 1;
     if (splits_override > 0) {
         splits = splits_override;
-    } else {
-        // fill the 256 compute units, keep at least 4 K groups per workgroup
-        while (tiles * splits < 256 && G / (splits * 2) >= 4 && splits < 64) splits *= 2;
+    } else if (p.mtiles == 1 && tiles < 256) {
+        double best = G * 0.7;
+        for (int sp = 2; sp <= 16; sp *= 2) {
+            if (G / sp < 4 || tiles * sp > 1024) break;
+            const double cost = (double)ceil_div_i(G, sp) * 0.7 + (double)m * n * sp / 150e3 + 5.0;
+            if (cost < best) {
+                best = cost;
+                splits = sp;
+            }
+        }
     }
     if (splits > G) splits = G;
     if (splits > 255) splits = 255;
