@@ -23,7 +23,7 @@
 //     sg ^ (r % 16);
 //   * per wave, its two packed rows of the strip (2 x 1 KiB): piece (c8, ch, kq) at position
 //     c8 + 8 ch + 16 kq, so a half-wave's 8-byte reads sweep all 64 banks;
-//   * per wave, the 256 bytes of scales of the strip.
+//   * per wave, the 256 bytes of scales of the strip (four copies, one per quarter-wave).
 // vmcnt is counted by hand: every stage issues exactly kStageOps LDS-DMA operations per
 // wave and nothing else uses the counter inside the loop.
 //
@@ -66,7 +66,7 @@ struct TileLds {
     static constexpr int kRows = 32 * MT;
     static constexpr int kXDwords = kRows * 64;        // X tile
     static constexpr int kBDwords = 4 * 2 * 256;       // 4 waves x 2 packed rows x 1 KiB
-    static constexpr int kSDwords = 4 * 64;            // 4 waves x 256 bytes of scales
+    static constexpr int kSDwords = 4 * 256;           // 4 waves x 4 copies of the strip's 256 bytes of scales
     static constexpr int kStageDwords = kXDwords + kBDwords + kSDwords;
     static constexpr size_t kRingBytes = (size_t)kRing * kStageDwords * 4;
     static constexpr size_t kRedBytes = (size_t)4 * 32 * 132 * 4;  // 4 waves x one 32-row M tile, fp32, padded rows
@@ -113,6 +113,7 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     const u32x4* strip_w = a.B + (size_t)strip * 64 + (size_t)w * N4;  // uniform; the lane adds piece_off
     // scales: lanes 0..15 fetch the 16 pieces (8 halves each) of the strip's 128 columns
     const half_t* strip_s = a.S + (size_t)strip * 128;  // uniform; the lane adds 8 * dslot
+    const int scale_row_stride = a.per_column ? 0 : a.N;  // per-column mode re-reads row 0 (unused)
 
     // X tile: wave w brings rows [kXOps 4 w, kXOps 4 (w+1)); one DMA instruction covers 4 rows
     // (64 lanes x 16 bytes, contiguous in LDS).  Lane l lands at row l/16, position l%16, so
@@ -170,9 +171,11 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
             __builtin_amdgcn_global_load_lds((gptr_t)(rowp + piece_off), (lptr_t)bbuf, 16, 0, 0);
         } else {
             // scales of the group (row 0 in per-column mode, unused then)
-            uint32_t* sbuf = stage + L::kXDwords + L::kBDwords + w * 64;
-            const half_t* ssrc = strip_s + (a.per_column ? (size_t)0 : (size_t)g * a.N);
-            if (dkq == 0) __builtin_amdgcn_global_load_lds((gptr_t)(ssrc + 8 * dslot), (lptr_t)sbuf, 16, 0, 0);
+            // all 64 lanes take part (a predicated load would split the loop body into several
+            // scheduling regions): the four quarter-waves fetch the same 256 bytes
+            uint32_t* sbuf = stage + L::kXDwords + L::kBDwords + w * 256;
+            const half_t* ssrc = strip_s + (size_t)g * scale_row_stride;
+            __builtin_amdgcn_global_load_lds((gptr_t)(ssrc + 8 * dslot), (lptr_t)sbuf, 16, 0, 0);
         }
     };
     auto issue_stage = [&](int g, int ring) __attribute__((always_inline)) {
@@ -201,7 +204,7 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     auto read_words = [&](int set, int ring) __attribute__((always_inline)) {
         const uint32_t* stage = lds + ring * L::kStageDwords;
         const uint32_t* bbuf = stage + L::kXDwords + w * 512;
-        const u32x2 sc_lds = *reinterpret_cast<const u32x2*>(stage + L::kXDwords + L::kBDwords + w * 64 + soff);
+        const u32x2 sc_lds = *reinterpret_cast<const u32x2*>(stage + L::kXDwords + L::kBDwords + w * 256 + soff);
         scv[set] = a.per_column ? sc_fixed : sc_lds;
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
@@ -219,40 +222,56 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
             xa[mt] = h8{d0.x, d0.y, d1.x, d1.y, d2.x, d2.y, d3.x, d3.y};
         }
     };
-    auto expand = [&](int set, int block) __attribute__((always_inline)) -> h8 {  // block = 4 t + 2 jo + blk
+    // One quarter (two of the eight values) of B operand `block` = 4 t + 2 jo + blk of a stage.
+    // K order of the operand: 4h, 4h+1 | 4h+2, 4h+3 | 4h+8, 4h+9 | 4h+10, 4h+11, i.e. quarter
+    // q = 0, 1: low-nibble form of pieces kq = 2h, 2h+1; q = 2, 3: high-nibble form.
+    auto expand_quarter = [&](int set, int block, int q) __attribute__((always_inline)) -> h2 {
         const int t = block >> 2, jo = (block >> 1) & 1, blk = block & 1;
         const h2 pr = bits_to_h2(scv[set][jo]);
-        const uint32_t q0 = blk ? (pw[set][t][0][jo] >> 8) : pw[set][t][0][jo];
-        const uint32_t q1 = blk ? (pw[set][t][1][jo] >> 8) : pw[set][t][1][jo];
+        const uint32_t word = pw[set][t][q & 1][jo];
+        const uint32_t qq = blk ? (word >> 8) : word;
         const h2 sv = blk ? h2{pr.y, pr.y} : h2{pr.x, pr.x};
-        // K order of the operand: 4h, 4h+1 | 4h+2, 4h+3 | 4h+8, 4h+9 | 4h+10, 4h+11
-        const h2 e0 = magic.pair_low(q0) * sv, e1 = magic.pair_low(q1) * sv;
-        const h2 e2 = magic.pair_high(q0) * sv, e3 = magic.pair_high(q1) * sv;
+        return (q < 2 ? magic.pair_low(qq) : magic.pair_high(qq)) * sv;
+    };
+    auto expand = [&](int set, int block) __attribute__((always_inline)) -> h8 {
+        const h2 e0 = expand_quarter(set, block, 0), e1 = expand_quarter(set, block, 1);
+        const h2 e2 = expand_quarter(set, block, 2), e3 = expand_quarter(set, block, 3);
         return h8{e0.x, e0.y, e1.x, e1.y, e2.x, e2.y, e3.x, e3.y};
     };
-    // Four of the eight blocks of a stage (2 packed rows x 4 B operands, MT MFMAs each).  The
-    // expansion of the following block is written between the MFMAs of a block, and so are
-    // the LDS-DMA loads of group next_g (first half only); the scheduler is told to keep that
-    // interleaving, because with one wave per SIMD nothing else fills the matrix pipe's shadow.
-    auto half_stage = [&](int set, int t, h8 (&xa)[MT], h8& bw, bool with_dma, int next_g, int next_ring) __attribute__((always_inline)) {
+    // Four of the eight blocks of a stage (2 packed rows x 4 B operands, MT MFMAs each), written
+    // as 4 MT slots: one MFMA, the share of the NEXT block's expansion that fits its shadow
+    // (4 / MT quarters), one LDS-DMA load of group next_g (first half only) and the LDS reads
+    // the caller assigns to the slot.  A scheduling barrier closes every slot: with one wave
+    // per SIMD nothing else fills the matrix pipe's shadow, so the order is fixed by hand.
+    auto half_stage = [&](int t, h8 (&xa)[MT], h8& bw, bool with_dma, int next_g, int next_ring, auto&& lds_reads) __attribute__((always_inline)) {
 #pragma unroll
         for (int op = 0; op < 4; ++op) {
             const int block = 4 * t + op;
-            const h8 bw_next = block < 7 ? expand(set, block + 1) : expand(set ^ 1, 0);
+            const int nset = block < 7 ? 0 : 1, nblock = block < 7 ? block + 1 : 0;
+            h2 e[4];
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt)
+            for (int mt = 0; mt < MT; ++mt) {
+                const int slot_i = op * MT + mt;
                 acc[mt][op] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xa[mt], bw, acc[mt][op], 0, 0, 0);
-            if (with_dma) {
 #pragma unroll
-                for (int idx = op; idx < kStageOps; idx += 4) issue_piece(next_g, next_ring, idx);
+                for (int q = mt * (4 / MT); q < (mt + 1) * (4 / MT); ++q) {
+                    // the empty asm pins the quarter to this slot: it cannot sink below the slot's
+                    // closing barrier
+                    uint32_t bits = h2_to_bits(expand_quarter(nset, nblock, q));
+                    asm volatile("" : "+v"(bits));
+                    e[q] = bits_to_h2(bits);
+                }
+                if (with_dma) {
+                    if (slot_i < kStageOps) issue_piece(next_g, next_ring, slot_i);
+                    if (slot_i == 0) {
+#pragma unroll
+                        for (int idx = 4 * MT; idx < kStageOps; ++idx) issue_piece(next_g, next_ring, idx);
+                    }
+                }
+                lds_reads(slot_i);
+                __builtin_amdgcn_sched_barrier(0);
             }
-            bw = bw_next;
-        }
-#pragma unroll
-        for (int i = 0; i < 4 * MT; ++i) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // 1 MFMA
-            __builtin_amdgcn_sched_group_barrier(0x002, MT == 4 ? 4 : (MT == 2 ? 8 : 16), 0);  // VALU
-            if (with_dma && i % 2 == 0) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);  // 1 VMEM read
+            bw = h8{e[0].x, e[0].y, e[1].x, e[1].y, e[2].x, e[2].y, e[3].x, e[3].y};
         }
     };
 
@@ -266,6 +285,13 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     // that every wave has finished reading the ring slot that the next iteration's loads
     // overwrite.  Past the end the "next" group is the last one again (loaded into a slot
     // nobody reads): no branches in the loop body and constant vmcnt arithmetic.
+    auto read_xa_one = [&](h8 (&xa)[MT], int ring, int t, int mt) __attribute__((always_inline)) {
+        const uint32_t* stage = lds + ring * L::kStageDwords;
+        const u32x2 lo = *reinterpret_cast<const u32x2*>(stage + mt * 2048 + xoff[t][0]);
+        const u32x2 hi = *reinterpret_cast<const u32x2*>(stage + mt * 2048 + xoff[t][1]);
+        const h2 d0 = bits_to_h2(lo.x), d1 = bits_to_h2(lo.y), d2 = bits_to_h2(hi.x), d3 = bits_to_h2(hi.y);
+        xa[mt] = h8{d0.x, d0.y, d1.x, d1.y, d2.x, d2.y, d3.x, d3.y};
+    };
     const int g_last = g_end - 1;
     h8 bw;
     if (ngroups > 0) {
@@ -282,13 +308,15 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
         const int slot_next = slot + 1 == kRing ? 0 : slot + 1;
         const int slot_refill = slot_next + 1 == kRing ? 0 : slot_next + 1;
         const int next_g = g_begin + it + 2 < g_end ? g_begin + it + 2 : g_last;
-        read_xa(xa1, slot, 1);
-        half_stage(0, 0, xa0, bw, true, next_g, slot_refill);
+        half_stage(0, xa0, bw, true, next_g, slot_refill, [&](int i) __attribute__((always_inline)) {
+            if (i < MT) read_xa_one(xa1, slot, 1, i);
+        });
         UNIQL_WAIT_VMCNT(kStageOps);   // stage it+1 has landed; only stage it+2's loads are outstanding
         __builtin_amdgcn_s_barrier();
-        read_words(1, slot_next);
-        read_xa(xa0, slot_next, 0);
-        half_stage(0, 1, xa1, bw, false, 0, 0);
+        half_stage(1, xa1, bw, false, 0, 0, [&](int i) __attribute__((always_inline)) {
+            if (i == 0) read_words(1, slot_next);
+            if (i >= 1 && i <= MT) read_xa_one(xa0, slot_next, 0, i - 1);
+        });
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
             pw[0][t][0] = pw[1][t][0];
