@@ -16,8 +16,9 @@
 // (two 8-byte LDS reads).
 //
 // Everything a group needs travels global -> LDS with global_load_lds_dwordx4 (no staging
-// registers) into a ring of three stages; the loads of group g+2 are issued while group g
-// is multiplied, and the operands of group g+1 are read from LDS into a second register set
+// registers) into a ring of three stages; the loads of group g+3 are issued during the second
+// half of group g, into the slot group g has just left, and the operands of group g+1 are read
+// from LDS into a second register set
 // during the second half of group g.  A stage holds
 //   * the X tile, 256 bytes per row, unpadded: 16-byte segment sg of row r sits at position
 //     sg ^ (r % 16);
@@ -240,10 +241,13 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     };
     // Four of the eight blocks of a stage (2 packed rows x 4 B operands, MT MFMAs each), written
     // as 4 MT slots: one MFMA, the share of the NEXT block's expansion that fits its shadow
-    // (4 / MT quarters), one LDS-DMA load of group next_g (first half only) and the LDS reads
-    // the caller assigns to the slot.  A scheduling barrier closes every slot: with one wave
+    // (4 / MT quarters), at most one LDS-DMA load (pieces dma_first.. of group next_g, one every
+    // kDmaStride slots: the four waves together must not outrun the compute unit's address
+    // path, or they stall at issue and the matrix pipe starves) and the LDS reads the caller
+    // assigns to the slot.  A scheduling barrier closes every slot: with one wave
     // per SIMD nothing else fills the matrix pipe's shadow, so the order is fixed by hand.
-    auto half_stage = [&](int t, h8 (&xa)[MT], h8& bw, bool with_dma, int next_g, int next_ring, auto&& lds_reads) __attribute__((always_inline)) {
+    auto half_stage = [&](int t, h8 (&xa)[MT], h8& bw, int dma_first, int dma_count, int next_g, int next_ring, auto&& lds_reads) __attribute__((always_inline)) {
+        constexpr int kDmaStride = MT == 1 ? 1 : 2;  // slots between two LDS-DMA loads
 #pragma unroll
         for (int op = 0; op < 4; ++op) {
             const int block = 4 * t + op;
@@ -261,14 +265,16 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
                     asm volatile("" : "+v"(bits));
                     e[q] = bits_to_h2(bits);
                 }
-                if (with_dma) {
-                    if (slot_i < kStageOps) issue_piece(next_g, next_ring, slot_i);
-                    if (slot_i == 0) {
-#pragma unroll
-                        for (int idx = 4 * MT; idx < kStageOps; ++idx) issue_piece(next_g, next_ring, idx);
-                    }
-                }
+                if (slot_i % kDmaStride == 0 && slot_i / kDmaStride < dma_count)
+                    issue_piece(next_g, next_ring, dma_first + slot_i / kDmaStride);
                 lds_reads(slot_i);
+                if (MT == 4) {
+                    // inside the slot: the first two operations of the quarter, the MFMA, the rest;
+                    // the MFMA between the fp16 add and the dependent multiply fills the wait
+                    // state that would otherwise cost an s_nop
+                    __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                }
                 __builtin_amdgcn_sched_barrier(0);
             }
             bw = h8{e[0].x, e[0].y, e[1].x, e[1].y, e[2].x, e[2].y, e[3].x, e[3].y};
@@ -277,14 +283,19 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
 
     // ---- software pipeline over the K groups ----------------------------------------------
     // Iteration `it` multiplies stage `it`.  First half: packed row w (A operands xa0), while
-    // the LDS-DMA loads of stage it+2 are issued and the A operands of packed row w+4 are
-    // read from LDS.  Middle: the wave waits for stage it+1 (only the loads just issued may
-    // remain outstanding) and the workgroup meets at a barrier.  Second half: packed row w+4
-    // (xa1), while the words, scales and first-row A operands of stage it+1 are read from LDS.
-    // So the matrix pipe never waits for the barrier or for LDS.  The barrier also guarantees
-    // that every wave has finished reading the ring slot that the next iteration's loads
-    // overwrite.  Past the end the "next" group is the last one again (loaded into a slot
-    // nobody reads): no branches in the loop body and constant vmcnt arithmetic.
+    // the A operands of packed row w+4 are read from LDS: after that nothing of stage `it` is
+    // left in LDS that anybody needs.  Middle: the wave waits for stage it+1 (only the kStageOps
+    // loads issued since may remain outstanding) and the workgroup meets at a barrier.  Second
+    // half: packed row w+4 (xa1), while the words, scales and first-row A operands of stage it+1
+    // are read from LDS.  The LDS-DMA loads of a stage are spread over a whole iteration: the
+    // first kDmaA pieces of stage it+3 go out in the second half of iteration it (into the
+    // slot stage `it` has just left), the rest in the first half of iteration it+1.  So the
+    // address path sees an even load, a piece has more than an iteration to land, and the matrix
+    // pipe never waits for the barrier or for LDS.  Past the end the "next" group is the last
+    // one again (loaded into a slot nobody reads): no branches in the loop body and constant
+    // vmcnt arithmetic.
+    constexpr int kDmaA = (kStageOps + 1) / 2, kDmaB = kStageOps - kDmaA;
+    auto group_or_last = [&](int g) __attribute__((always_inline)) { return g < g_end ? g : g_end - 1; };
     auto read_xa_one = [&](h8 (&xa)[MT], int ring, int t, int mt) __attribute__((always_inline)) {
         const uint32_t* stage = lds + ring * L::kStageDwords;
         const u32x2 lo = *reinterpret_cast<const u32x2*>(stage + mt * 2048 + xoff[t][0]);
@@ -297,7 +308,9 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     if (ngroups > 0) {
         issue_stage(g_begin, 0);
         issue_stage(ngroups > 1 ? g_begin + 1 : g_last, 1);
-        UNIQL_WAIT_VMCNT(kStageOps);
+#pragma unroll
+        for (int idx = 0; idx < kDmaA; ++idx) issue_piece(group_or_last(g_begin + 2), 2, idx);
+        UNIQL_WAIT_VMCNT(kStageOps + kDmaA);
         __builtin_amdgcn_s_barrier();
         read_words(0, 0);
         read_xa(xa0, 0, 0);
@@ -306,14 +319,13 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     int slot = 0;
     for (int it = 0; it < ngroups; ++it) {
         const int slot_next = slot + 1 == kRing ? 0 : slot + 1;
-        const int slot_refill = slot_next + 1 == kRing ? 0 : slot_next + 1;
-        const int next_g = g_begin + it + 2 < g_end ? g_begin + it + 2 : g_last;
-        half_stage(0, xa0, bw, true, next_g, slot_refill, [&](int i) __attribute__((always_inline)) {
+        const int slot_prev = slot == 0 ? kRing - 1 : slot - 1;   // holds stage it+2
+        half_stage(0, xa0, bw, kDmaA, kDmaB, group_or_last(g_begin + it + 2), slot_prev, [&](int i) __attribute__((always_inline)) {
             if (i < MT) read_xa_one(xa1, slot, 1, i);
         });
         UNIQL_WAIT_VMCNT(kStageOps);   // stage it+1 has landed; only stage it+2's loads are outstanding
         __builtin_amdgcn_s_barrier();
-        half_stage(1, xa1, bw, false, 0, 0, [&](int i) __attribute__((always_inline)) {
+        half_stage(1, xa1, bw, 0, kDmaA, group_or_last(g_begin + it + 3), slot, [&](int i) __attribute__((always_inline)) {
             if (i == 0) read_words(1, slot_next);
             if (i >= 1 && i <= MT) read_xa_one(xa0, slot_next, 0, i - 1);
         });
