@@ -10,10 +10,12 @@
 // Operand layout.  A 16-byte piece (c8, kq) of a packed row holds, in 32-bit word j,
 // K rows {2kq, 2kq+1, 2kq+8, 2kq+9} of columns 16j + c8 and 16j + 8 + c8.  Lane
 //     l = s + 32 h,  s = c8 + 8 ch + 16 jl      (ch: 64-column chunk of the strip)
-// reads words 2jl, 2jl+1 of the pieces kq = 2h and 2h+1 and builds four B operands
-// (jo, blk): column 64 ch + 16 (2jl + jo) + 8 blk + c8, K values {4h..4h+3, 4h+8..4h+11}.
-// The A operand of a 32-row M tile is row l % 32 of X with the same eight K values
-// (two 8-byte LDS reads).
+// reads words 2jl, 2jl+1 of the pieces kq = 2h and 2h+1 and builds four weight operands
+// (jo, blk): column 64 ch + 16 (2jl + jo) + 8 blk + c8, K values {4h..4h+3, 4h+8..4h+11}
+// (called B operands below).  The activation operand of a 32-row M tile (called A operand) is
+// row l % 32 of X with the same eight K values (two 8-byte LDS reads).  The MFMA gets the
+// weights as its first source and the activations as its second: the product comes out
+// transposed, which gives every lane four consecutive output columns per register quad.
 //
 // Everything a group needs travels global -> LDS with global_load_lds_dwordx4 (no staging
 // registers) into a ring of three stages; the loads of group g+3 are issued during the second
@@ -256,7 +258,7 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 const int slot_i = op * MT + mt;
-                acc[mt][op] = __builtin_amdgcn_mfma_f32_32x32x16_f16(xa[mt], bw, acc[mt][op], 0, 0, 0);
+                acc[mt][op] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bw, xa[mt], acc[mt][op], 0, 0, 0);
 #pragma unroll
                 for (int q = mt * (4 / MT); q < (mt + 1) * (4 / MT); ++q) {
                     // the empty asm pins the quarter to this slot: it cannot sink below the slot's
@@ -341,11 +343,13 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     __syncthreads();
 
     // ---- add the four waves' partial tiles, one 32-row M tile at a time ---------------------
-    // acc[mt][2 jo + blk][v] on lane l: row 32 mt + 8 (v / 4) + 4 h + v % 4,
-    // column 64 ch + 16 (2 jl + jo) + 8 blk + c8 of the strip.  Every wave writes its partial
-    // tile to LDS (row stride 132 floats: rows 4 apart fall on different banks); then each
-    // thread adds the four partials of two (row, 8 consecutive columns) units and stores
-    // each unit with one 16-byte store.
+    // The MFMAs take the weights as their first operand, so the accumulators hold the tile
+    // transposed: acc[mt][2 jo + blk][4 j4 + i] on lane l is row 32 mt + l % 32 of the tile and
+    // column 64 (j4 % 2) + 16 (2 (j4 / 2) + jo) + 8 blk + 4 h + i of the strip, i.e. four
+    // consecutive columns per group of four registers: one 16-byte LDS write each.  Every wave
+    // writes its partial tile to LDS (row stride 132 floats); then each thread adds the four
+    // partials of two (row, 8 consecutive columns) units and stores each unit with one 16-byte
+    // store.
     constexpr int kRedStride = 132;
     float* red = reinterpret_cast<float*>(lds);  // [4 waves][32 rows][132]
     const bool split_k = a.splits > 1;
@@ -354,12 +358,13 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
         if (m0 + mt * 32 < a.M) {  // uniform
             if (mt > 0) __syncthreads();
             {
-                float* wred = red + w * 32 * kRedStride + (4 * h) * kRedStride + 64 * ch + 32 * jl + c8;
+                float* wred = red + w * 32 * kRedStride + s * kRedStride + 4 * h;
 #pragma unroll
                 for (int op = 0; op < 4; ++op)
 #pragma unroll
-                    for (int v = 0; v < 16; ++v)
-                        wred[(8 * (v >> 2) + (v & 3)) * kRedStride + 16 * (op >> 1) + 8 * (op & 1)] = acc[mt][op][v];
+                    for (int j4 = 0; j4 < 4; ++j4)
+                        *reinterpret_cast<f4*>(wred + 64 * (j4 & 1) + 32 * (j4 >> 1) + 16 * (op >> 1) + 8 * (op & 1)) =
+                            f4{acc[mt][op][4 * j4], acc[mt][op][4 * j4 + 1], acc[mt][op][4 * j4 + 2], acc[mt][op][4 * j4 + 3]};
             }
             __syncthreads();
             if (!split_k) {
