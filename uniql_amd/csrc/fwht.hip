@@ -94,6 +94,120 @@ __global__ __launch_bounds__(256) void fwht_lds_kernel(const T* __restrict__ x, 
     }
 }
 
+// ---- fp16, power of two >= 256: vector loads, index bits 0..2 in registers, LDS passes of
+// up to four bits, vector stores --------------------------------------------------------
+// The fp32 image in LDS is padded by eight floats per 128: in the first LDS pass (bits 3..6)
+// the lanes of a wave differ in bits 0..2 and 7.., and the padding moves each step of bit 7
+// to another group of eight banks; the later passes walk consecutive addresses anyway.
+__device__ __forceinline__ int fwht_pad(int idx) { return idx + ((idx >> 7) << 3); }
+
+template <int CNT>
+__device__ __forceinline__ void fwht_pass_padded(float* buf, int L, int lo, int tid, int nthreads) {
+    constexpr int E = 1 << CNT;
+    const int tasks = L >> CNT;
+    const int lowmask = (1 << lo) - 1;
+    for (int t = tid; t < tasks; t += nthreads) {
+        const int base = ((t >> lo) << (lo + CNT)) | (t & lowmask);
+        float v[E];
+#pragma unroll
+        for (int i = 0; i < E; ++i) v[i] = buf[fwht_pad(base + (i << lo))];
+#pragma unroll
+        for (int h = 1; h < E; h <<= 1) {
+#pragma unroll
+            for (int i = 0; i < E; ++i) {
+                if ((i & h) == 0) {
+                    const float p = v[i], q = v[i + h];
+                    v[i] = p + q;
+                    v[i + h] = p - q;
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < E; ++i) buf[fwht_pad(base + (i << lo))] = v[i];
+    }
+}
+
+__global__ __launch_bounds__(1024) void fwht_f16_kernel(const u32x4* __restrict__ x, u32x4* __restrict__ y, int L,
+                                                       int log2L, float scale) {
+    extern __shared__ __attribute__((aligned(16))) float fbuf[];
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int chunks = L >> 3;
+    const u32x4* xp = x + (size_t)blockIdx.x * chunks;
+    u32x4* yp = y + (size_t)blockIdx.x * chunks;
+    for (int c = tid; c < chunks; c += nthreads) {
+        const u32x4 v = xp[c];
+        float f[8];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const h2 hv = bits_to_h2(v[p]);
+            f[2 * p] = (float)hv.x;
+            f[2 * p + 1] = (float)hv.y;
+        }
+#pragma unroll
+        for (int h = 1; h < 8; h <<= 1) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                if ((i & h) == 0) {
+                    const float p = f[i], q = f[i + h];
+                    f[i] = p + q;
+                    f[i + h] = p - q;
+                }
+            }
+        }
+        float* dst = fbuf + fwht_pad(8 * c);
+        *reinterpret_cast<f4*>(dst) = f4{f[0], f[1], f[2], f[3]};
+        *reinterpret_cast<f4*>(dst + 4) = f4{f[4], f[5], f[6], f[7]};
+    }
+    __syncthreads();
+    int lo = 3;
+    while (lo < log2L) {
+        const int left = log2L - lo;
+        if (left >= 4) {
+            fwht_pass_padded<4>(fbuf, L, lo, tid, nthreads);
+            lo += 4;
+        } else if (left == 3) {
+            fwht_pass_padded<3>(fbuf, L, lo, tid, nthreads);
+            lo += 3;
+        } else if (left == 2) {
+            fwht_pass_padded<2>(fbuf, L, lo, tid, nthreads);
+            lo += 2;
+        } else {
+            fwht_pass_padded<1>(fbuf, L, lo, tid, nthreads);
+            lo += 1;
+        }
+        __syncthreads();
+    }
+    for (int c = tid; c < chunks; c += nthreads) {
+        const float* src = fbuf + fwht_pad(8 * c);
+        const f4 a = *reinterpret_cast<const f4*>(src), b = *reinterpret_cast<const f4*>(src + 4);
+        h2 r0, r1, r2, r3;
+        r0.x = scaled_to_half(a[0], scale);
+        r0.y = scaled_to_half(a[1], scale);
+        r1.x = scaled_to_half(a[2], scale);
+        r1.y = scaled_to_half(a[3], scale);
+        r2.x = scaled_to_half(b[0], scale);
+        r2.y = scaled_to_half(b[1], scale);
+        r3.x = scaled_to_half(b[2], scale);
+        r3.y = scaled_to_half(b[3], scale);
+        yp[c] = u32x4{h2_to_bits(r0), h2_to_bits(r1), h2_to_bits(r2), h2_to_bits(r3)};
+    }
+}
+
+static int fwht_f16_launch(const void* x, void* y, int64_t pieces, int block, float scale, hipStream_t stream) {
+    int log2L = 0;
+    while ((1 << log2L) < block) ++log2L;
+    const size_t shmem = (size_t)(block + (block >> 7) * 8) * sizeof(float);
+    if (shmem > 64 * 1024) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(&fwht_f16_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
+            return UNIQL_E_LAUNCH;
+    }
+    const int threads = block / 8 < 1024 ? block / 8 : 1024;
+    hipLaunchKernelGGL(fwht_f16_kernel, dim3((unsigned)pieces), dim3(threads), shmem, stream,
+                       reinterpret_cast<const u32x4*>(x), reinterpret_cast<u32x4*>(y), block, log2L, scale);
+    return UNIQL_OK;
+}
+
 template <typename T>
 static int fwht_lds_launch(const void* x, void* y, int64_t pieces, int block, float scale, hipStream_t stream) {
     int log2L = 0;
@@ -121,7 +235,8 @@ int fwht_launch(const void* x, void* y, int64_t rows, int dim, int block, float 
     } else {
         if (pieces > 0x7fffffffLL) return UNIQL_E_SHAPE;
         int rc;
-        if (dtype == UNIQL_DT_F16) rc = fwht_lds_launch<half_t>(x, y, pieces, block, scale, stream);
+        if (dtype == UNIQL_DT_F16 && block >= 256) rc = fwht_f16_launch(x, y, pieces, block, scale, stream);
+        else if (dtype == UNIQL_DT_F16) rc = fwht_lds_launch<half_t>(x, y, pieces, block, scale, stream);
         else if (dtype == UNIQL_DT_BF16) rc = fwht_lds_launch<__bf16>(x, y, pieces, block, scale, stream);
         else rc = fwht_lds_launch<float>(x, y, pieces, block, scale, stream);
         if (rc != UNIQL_OK) return rc;
