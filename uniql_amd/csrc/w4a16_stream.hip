@@ -368,19 +368,28 @@ struct StreamPlan {
     int waves;  // 4, 8 or 16
     int upw;    // groups per wave
     int splits;
+    bool prefetch;
 };
 
-// Heuristic: shapes with enough strips to occupy the chip on their own let one workgroup
-// of 16 waves own a whole strip (no exchange of partial sums); otherwise K is split
-// over workgroups of 4 waves.
+// Heuristic (from sweeps over waves x groups per wave on the Llama shapes): shapes with enough
+// strips to occupy the chip on their own let one workgroup own a whole strip, so no partial
+// sums are exchanged: 8 waves without the second register set (two workgroups per compute
+// unit) for one or two rows, 16 waves for more rows; otherwise K is split over workgroups of
+// 4 waves, or of 8 when that still leaves fewer than three waves per SIMD.
 static StreamPlan stream_plan(int m, int n, int k, int upw_override, int waves_override) {
     const int nstrips = n / 128, G = k / 128;
     StreamPlan p;
     p.waves = 4;
+    p.prefetch = true;
+    const bool whole_strip = m <= 16 && nstrips >= 192 && G >= 16 && G <= 64;
     if (waves_override) p.waves = waves_override;
-    else if (m <= 16 && nstrips >= 192 && G >= 16) p.waves = 16;
+    else if (whole_strip) p.waves = m <= 2 ? 8 : 16;
+    else if (m <= 2 && (int64_t)nstrips * G >= 1536 && (int64_t)nstrips * G < 3072) p.waves = 8;
     if (upw_override > 0) {
         p.upw = upw_override;
+    } else if (whole_strip && !waves_override) {
+        p.upw = ceil_div(G, p.waves);
+        p.prefetch = false;
     } else if (p.waves == 16) {
         p.upw = ceil_div(G, 16);
         if (p.upw > 8) p.upw = 8;
@@ -471,7 +480,7 @@ int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void
         a.xrows = mt == 1 ? ((mm + 3) / 4) * 4 : mt * 16;
         a.X = reinterpret_cast<const half_t*>(A) + (size_t)m0 * lda;
         a.D = reinterpret_cast<char*>(D) + (size_t)m0 * n * out_elt;
-        const bool pf = !(tune & 0x2000u) && plan.upw > 1 && plan.waves != 16;
+        const bool pf = !(tune & 0x2000u) && plan.prefetch && plan.upw > 1 && plan.waves != 16;
         const hipError_t e = had128 ? launch_rows<true>(a, mt, plan.waves, pf, stream)
                                     : launch_rows<false>(a, mt, plan.waves, pf, stream);
         if (e != hipSuccess) return UNIQL_E_LAUNCH;
