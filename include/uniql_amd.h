@@ -105,6 +105,39 @@ int uniql_w4a16_dequant(const void* B, const void* S, void* W, uint8_t* codes,
                         int n, int k, int groups, void* stream);
 
 /*
+ * Group-128 quantisation of an fp16 weight matrix on the device, straight into the packed
+ * layout.  Replaces the host arithmetic of W4A16B16O16Linear.from_fp16
+ * (quantize/quant_linear_layers.py:50-89 -> quantize/quantize_helpers.py:87-141,183-241: fp16
+ * tensors on the CPU, every operation rounded to fp16) with the same results bit for bit.
+ *   W             device, fp16 [out_features, in_features] row-major (nn.Linear.weight), row
+ *                 stride ldw elements
+ *   given_scales  NULL: scale = fp16(max|w| * 2/15) per (group of 128 K, column), code =
+ *                 clamp(round(w / scale) + 8, 0, 15).  Otherwise device fp16
+ *                 [k_pad/128, out_features], natural order: the GPTQ hand-over
+ *                 (quantize_helpers.py:205-218), code = clamp(round(w / scale + 8), 0, 15)
+ *   B             device out, int32 [k_pad/16, 2 n_pad]
+ *   S             device out, fp16 [k_pad/128, n_pad], permuted
+ *   k_pad = in_features rounded up to 128 (rows past in_features count as zero weights),
+ *   n_pad >= out_features, n_pad % 128 == 0 (columns past out_features get code 0, scale 0);
+ *   in_features > 128 (the one-scale-per-column case of the reference is not produced).
+ */
+int uniql_w4a16_quantize(const void* W, int64_t ldw, const void* given_scales, void* B, void* S,
+                         int out_features, int in_features, int n_pad, int k_pad, void* stream);
+
+/*
+ * Packs ready codes and natural-order scales: the inverse of uniql_w4a16_dequant's `codes`
+ * output.  Replaces get_w4a16_permute_weights + w4a16_permute_scales
+ * (quantize/quantize_helpers.py:66-84,168-180) as the slicing functions of
+ * modeling/modeling_helpers.py:235-867 use them after cutting the unpacked tensors.
+ *   codes   device, uint8 [k, n] (values 0..15)
+ *   scales  device, fp16 [k/128, n], natural order
+ *   B       device out, int32 [k/16, 2 n_pad];  S  device out, fp16 [k/128, n_pad], permuted
+ *   k % 128 == 0, n_pad >= n, n_pad % 128 == 0 (padding columns: code 0, scale 0)
+ */
+int uniql_w4a16_pack(const uint8_t* codes, const void* scales, void* B, void* S, int n, int k, int n_pad,
+                     void* stream);
+
+/*
  * out[t, :] = fp16_rn((code - 8) * scales[ids[t]]) for t < ntokens.
  * Replaces quant_embedding_cuda.w4a16_embedding_lookup
  * (csrc/embedding/quant_embedding_kernel.cuh:80-166).

@@ -1,0 +1,116 @@
+"""Producer side on the GPU: quantise + pack (uniql_w4a16_quantize), pack ready codes
+(uniql_w4a16_pack) and the unpack -> slice -> repack round trip, against the reference's own
+outputs (golden fixtures) and the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import uniql_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("case,pad_out", [("A", 0), ("B", 192), ("C", 0)])
+def test_quantize_matches_reference_vectors(gpu, golden, case, pad_out):
+    """w4a16_quantize of the reference on seeded matrices: plain, N padded by 192, K padded with
+    an all-zero group (the fixtures hold the reference's packed words and permuted scales)."""
+    from uniql_amd import ops
+    w_kn = torch.from_numpy(golden[f"{case}_w"])                    # [K, N] as the reference takes it
+    packed, scale = ops.w4a16_quantize(w_kn.t().contiguous().to(gpu), None, pad_out=pad_out)
+    assert np.array_equal(packed.cpu().numpy(), golden[f"{case}_packed"])
+    assert np.array_equal(scale.cpu().numpy().view(np.uint16), golden[f"{case}_scale"].view(np.uint16))
+
+
+def test_quantize_given_scales_matches_reference_vectors(gpu, golden):
+    """The GPTQ hand-over: codes re-derived from given scales (quantize_helpers.py:205-218)."""
+    from uniql_amd import ops
+    w = torch.from_numpy(golden["G_w"]).t().contiguous().to(gpu)
+    s_in = torch.from_numpy(golden["G_scale_in"]).to(gpu)
+    packed, scale = ops.w4a16_quantize(w, s_in)
+    assert np.array_equal(packed.cpu().numpy(), golden["G_packed"])
+    assert np.array_equal(scale.cpu().numpy().view(np.uint16), golden["G_scale"].view(np.uint16))
+
+
+@pytest.mark.parametrize("k,n,pad_out,spread", [(256, 256, 0, 0.05), (384, 320, 192, 1.0), (1000, 256, 0, 0.05),
+                                                (4096, 1024, 0, 0.02), (512, 128, 128, 1e-6)])
+def test_quantize_matches_oracle_on_random_weights(gpu, k, n, pad_out, spread):
+    """Bit for bit against the oracle (itself pinned to the fixtures above), including K that is
+    not a multiple of 128, weights small enough for subnormal scales, and exact zeros."""
+    from uniql_amd import ops
+    g = torch.Generator().manual_seed(k + n)
+    w = (torch.randn(n, k, generator=g) * spread).half()
+    w[::7, 5:9] = 0
+    if k >= 512:
+        w[3, 128:256] = 0                                           # an all-zero group
+    _, o_packed, o_scale = O.w4a16_quantize(w.t().contiguous(), 128, None, pad_out)
+    packed, scale = ops.w4a16_quantize(w.to(gpu), None, pad_out=pad_out)
+    assert torch.equal(packed.cpu(), o_packed)
+    assert np.array_equal(scale.cpu().numpy().view(np.uint16), o_scale.numpy().view(np.uint16))
+
+
+def test_quantize_strided_weight(gpu):
+    from uniql_amd import ops
+    g = torch.Generator().manual_seed(9)
+    big = (torch.randn(256, 512, generator=g) * 0.1).half().to(gpu)
+    view = big[:, :384]
+    a = ops.w4a16_quantize(view)
+    b = ops.w4a16_quantize(view.contiguous())
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+def test_pack_matches_reference_vectors(gpu, golden):
+    from uniql_amd import ops
+    codes = torch.from_numpy(golden["P_codes"]).to(gpu)
+    scales = torch.ones((1, codes.shape[1]), dtype=torch.float16, device=gpu)
+    packed, _ = ops.w4a16_pack(codes, scales)
+    assert np.array_equal(packed.cpu().numpy(), golden["P_packed"])
+    for case in ("A", "B", "C"):
+        codes = torch.from_numpy(golden[f"{case}_codes"]).to(gpu)
+        scales = torch.from_numpy(golden[f"{case}_scale_unperm"]).to(gpu)
+        packed, scale = ops.w4a16_pack(codes, scales)
+        assert np.array_equal(packed.cpu().numpy(), golden[f"{case}_packed"])
+        assert np.array_equal(scale.cpu().numpy().view(np.uint16), golden[f"{case}_scale"].view(np.uint16))
+
+
+def test_unpack_slice_repack(gpu):
+    """The reference's load-time slicing (modeling_helpers.py:235-355) unpacks, cuts columns or
+    whole K groups and packs again; the same on the device equals packing the cut tensors."""
+    from uniql_amd import ops
+    rng = np.random.default_rng(5)
+    k, n = 1024, 512
+    q = rng.integers(0, 16, size=(k, n)).astype(np.int32)
+    s = rng.uniform(0.004, 0.02, size=(k // 128, n)).astype(np.float16)
+    packed = torch.from_numpy(O.pack_weights(q)).to(gpu)
+    s_perm = torch.from_numpy(O.permute_scales(s, k, n, 128)).to(gpu)
+    codes, scales = ops.w4a16_unpack(packed, s_perm, n, k)
+    assert np.array_equal(codes.cpu().numpy(), q.astype(np.uint8))
+    assert np.array_equal(scales.cpu().numpy().view(np.uint16), s.view(np.uint16))
+    # keep 384 of the columns (an up/gate-style cut) ...
+    keep_n = np.sort(rng.choice(n, size=384, replace=False))
+    idx = torch.from_numpy(keep_n).to(gpu)
+    p2, s2 = ops.w4a16_pack(codes[:, idx], scales[:, idx])
+    assert np.array_equal(p2.cpu().numpy(), O.pack_weights(q[:, keep_n]))
+    assert np.array_equal(s2.cpu().numpy().view(np.uint16),
+                          O.permute_scales(s[:, keep_n], k, 384, 128).view(np.uint16))
+    # ... and 5 of the 8 K groups (a down-style cut), output columns padded to 256
+    groups = [0, 2, 3, 6, 7]
+    rows = np.concatenate([np.arange(128 * g, 128 * g + 128) for g in groups])
+    ridx = torch.from_numpy(rows).to(gpu)
+    gidx = torch.tensor(groups, device=gpu)
+    p3, s3 = ops.w4a16_pack(codes[ridx][:, idx], scales[gidx][:, idx], pad_out=128)
+    q_cut = np.concatenate([q[rows][:, keep_n], np.zeros((len(rows), 128), np.int32)], axis=1)
+    s_cut = np.concatenate([s[groups][:, keep_n], np.zeros((len(groups), 128), np.float16)], axis=1)
+    assert np.array_equal(p3.cpu().numpy(), O.pack_weights(q_cut))
+    assert np.array_equal(s3.cpu().numpy().view(np.uint16),
+                          O.permute_scales(s_cut, len(rows), 512, 128).view(np.uint16))
+
+
+def test_quantize_errors(gpu):
+    from uniql_amd import ops
+    with pytest.raises(RuntimeError):
+        ops.w4a16_quantize(torch.zeros(256, 128, dtype=torch.float16, device=gpu))      # in_features <= 128
+    with pytest.raises(RuntimeError):
+        ops.w4a16_quantize(torch.zeros(256, 256, dtype=torch.float32, device=gpu))
+    with pytest.raises(RuntimeError):
+        ops.w4a16_pack(torch.zeros(100, 128, dtype=torch.uint8, device=gpu),
+                       torch.zeros(0, 128, dtype=torch.float16, device=gpu))

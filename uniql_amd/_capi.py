@@ -28,6 +28,9 @@ SIGNATURES = {
                                  c_void_p, c_int64, c_void_p, c_size_t, c_void_p, c_size_t,
                                  c_int, c_int, c_int, c_int, c_int, c_float, c_uint, c_void_p]),
     "uniql_w4a16_dequant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
+    "uniql_w4a16_quantize": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
+                                     c_int, c_int, c_int, c_int, c_void_p]),
+    "uniql_w4a16_pack": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "uniql_w4_embedding_lookup": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
                                           c_int64, c_int, c_void_p]),
     "uniql_fwht": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_float, c_int, c_void_p]),

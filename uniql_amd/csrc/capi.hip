@@ -16,6 +16,10 @@ int embedding_launch(const int64_t* ids, int64_t ntokens, const void* weight, co
                      int64_t vocab, int dim, hipStream_t stream);
 int fwht_launch(const void* x, void* y, int64_t rows, int dim, int block, float scale, int dtype,
                 hipStream_t stream);
+int quantize_launch(const void* W, int64_t ldw, const void* given_scales, void* B, void* S, int out_features,
+                    int in_features, int n_pad, int k_pad, hipStream_t stream);
+int pack_launch(const uint8_t* codes, const void* scales, void* B, void* S, int n, int k, int n_pad, int k_pad,
+                hipStream_t stream);
 }  // namespace uniql
 
 using namespace uniql;
@@ -124,6 +128,25 @@ int uniql_w4a16_dequant(const void* B, const void* S, void* W, uint8_t* codes, i
     if (!B || !S || (!W && !codes)) return UNIQL_E_NULL;
     if (!aligned16(B)) return UNIQL_E_ALIGN;
     return dequant_launch(B, S, W, codes, n, k, groups, reinterpret_cast<hipStream_t>(stream));
+}
+
+int uniql_w4a16_quantize(const void* W, int64_t ldw, const void* given_scales, void* B, void* S, int out_features,
+                         int in_features, int n_pad, int k_pad, void* stream) {
+    if (!W || !B || !S) return UNIQL_E_NULL;
+    if (out_features <= 0 || in_features <= 0 || ldw < in_features) return UNIQL_E_SHAPE;
+    if (k_pad != (in_features + 127) / 128 * 128 || n_pad < out_features || n_pad % 128 != 0) return UNIQL_E_SHAPE;
+    if (in_features <= 128) return UNIQL_E_UNSUPPORTED;
+    if ((int64_t)(k_pad / 16) * 2 * n_pad > 0x7fffffffLL * 256) return UNIQL_E_SHAPE;
+    return quantize_launch(W, ldw, given_scales, B, S, out_features, in_features, n_pad, k_pad,
+                           reinterpret_cast<hipStream_t>(stream));
+}
+
+int uniql_w4a16_pack(const uint8_t* codes, const void* scales, void* B, void* S, int n, int k, int n_pad,
+                     void* stream) {
+    if (!codes || !scales || !B || !S) return UNIQL_E_NULL;
+    if (n <= 0 || k <= 0 || k % 128 != 0 || n_pad < n || n_pad % 128 != 0) return UNIQL_E_SHAPE;
+    if ((int64_t)(k / 16) * 2 * n_pad > 0x7fffffffLL * 256) return UNIQL_E_SHAPE;
+    return pack_launch(codes, scales, B, S, n, k, n_pad, k, reinterpret_cast<hipStream_t>(stream));
 }
 
 int uniql_w4_embedding_lookup(const int64_t* ids, int64_t ntokens, const void* weight, const void* scales,

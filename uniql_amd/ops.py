@@ -129,6 +129,68 @@ def w4a16_dequant(B: torch.Tensor, s: torch.Tensor, size_n: int, size_k: int, wa
     return (W, codes) if want_codes else W
 
 
+def w4a16_quantize(weight: torch.Tensor, given_scale: torch.Tensor | None = None, pad_out: int = 0):
+    """Group-128 quantisation of an nn.Linear weight [out_features, in_features] (fp16, on the
+    GPU) into (packed int32 [k_pad/16, 2 n_pad], permuted scale fp16 [k_pad/128, n_pad]), with the
+    host arithmetic of the reference's from_fp16 / w4a16_quantize bit for bit.  given_scale:
+    natural-order [k_pad/128, out_features] scales of already fake-quantised weights (GPTQ)."""
+    _require_gpu(weight, "weight")
+    if weight.dtype != torch.float16 or weight.dim() != 2 or weight.stride(1) != 1:
+        raise RuntimeError("weight must be float16 [out_features, in_features] with unit inner stride")
+    out_features, in_features = weight.shape
+    k_pad = (in_features + 127) // 128 * 128
+    n_pad = out_features + pad_out
+    dev = weight.device
+    if given_scale is not None:
+        _require_gpu(given_scale, "given_scale")
+        if given_scale.dtype != torch.float16 or tuple(given_scale.shape) != (k_pad // 128, out_features) \
+                or not given_scale.is_contiguous():
+            raise RuntimeError("given_scale must be contiguous float16 [k_pad/128, out_features]")
+    lib = _capi.load()
+    with torch.cuda.device(dev):
+        B = torch.empty((k_pad // 16, 2 * n_pad), dtype=torch.int32, device=dev)
+        S = torch.empty((k_pad // 128, n_pad), dtype=torch.float16, device=dev)
+        code = lib.uniql_w4a16_quantize(weight.data_ptr(), weight.stride(0),
+                                        given_scale.data_ptr() if given_scale is not None else None,
+                                        B.data_ptr(), S.data_ptr(), out_features, in_features, n_pad, k_pad,
+                                        _stream_ptr(dev))
+    _capi.check(code, "uniql_w4a16_quantize")
+    return B, S
+
+
+def w4a16_pack(codes: torch.Tensor, scales: torch.Tensor, pad_out: int = 0):
+    """codes uint8 [k, n] and natural-order scales fp16 [k/128, n] -> (packed, permuted scale);
+    the inverse of w4a16_unpack."""
+    _require_gpu(codes, "codes")
+    _require_gpu(scales, "scales")
+    if codes.dtype != torch.uint8 or scales.dtype != torch.float16 or codes.dim() != 2:
+        raise RuntimeError("codes must be uint8 [k, n] and scales float16 [k/128, n]")
+    k, n = codes.shape
+    if tuple(scales.shape) != (k // 128, n):
+        raise RuntimeError("scales must be [k/128, n]")
+    codes, scales = codes.contiguous(), scales.contiguous()
+    n_pad = n + pad_out
+    dev = codes.device
+    lib = _capi.load()
+    with torch.cuda.device(dev):
+        B = torch.empty((k // 16, 2 * n_pad), dtype=torch.int32, device=dev)
+        S = torch.empty((k // 128, n_pad), dtype=torch.float16, device=dev)
+        code = lib.uniql_w4a16_pack(codes.data_ptr(), scales.data_ptr(), B.data_ptr(), S.data_ptr(), n, k, n_pad,
+                                    _stream_ptr(dev))
+    _capi.check(code, "uniql_w4a16_pack")
+    return B, S
+
+
+def w4a16_unpack(B: torch.Tensor, s: torch.Tensor, size_n: int, size_k: int):
+    """(codes uint8 [k, n], natural-order scales fp16 [k/128, n]) of a packed group-128 layer:
+    what the reference's slicing code gets from unpack_w4a16_permute_weights and
+    w4a16_unpermute_scales (quantize_helpers.py:244-328) on the CPU."""
+    _, codes = w4a16_dequant(B, s, size_n, size_k, want_codes=True)
+    n = torch.arange(size_n, device=B.device)
+    pos = (n & ~63) + 8 * (n & 7) + ((n & 63) >> 3)
+    return codes, s[:, pos].contiguous()
+
+
 def w4a16_embedding_lookup(input: torch.Tensor, weight: torch.Tensor, scale: torch.Tensor) -> torch.Tensor:
     """out[..., :] = (code - 8) * scale[id].  Checks follow quant_embedding_kernel.cuh:121-134."""
     if weight.dim() != 2:

@@ -53,8 +53,10 @@ class W4A16B16O16Linear(nn.Module):
 
     @classmethod
     def from_fp16(cls, originalLayer: nn.Linear):
-        """Quantises an nn.Linear on the CPU in fp16 (the reference's arithmetic,
-        quant_linear_layers.py:50-89) and packs it for the kernel."""
+        """Quantises an nn.Linear in fp16 with the reference's arithmetic
+        (quant_linear_layers.py:50-89) and packs it for the kernel: on the GPU when the layer's
+        weight lives there (same results bit for bit), on the CPU otherwise as the reference
+        does."""
         group_size = 128 if originalLayer.in_features > 128 else -1
         given_scale = None
         if getattr(originalLayer, "apply_gptq", False):
@@ -67,6 +69,15 @@ class W4A16B16O16Linear(nn.Module):
         W = originalLayer.weight
         dev = W.device
         q = cls(originalLayer.in_features, originalLayer.out_features, device=dev)
+        if W.is_cuda and group_size == 128:
+            w16 = W.detach().to(torch.float16).contiguous()                # [Dout, Din]
+            scale_dev = None if given_scale is None else given_scale.to(dev).contiguous()
+            q.weight, q.scale = ops.w4a16_quantize(w16, scale_dev, pad_out=q.pad_out)
+            q.size_k, q.size_n = q.weight.shape[0] * 16, q.weight.shape[1] // 2
+            q.pad_in = q.size_k - originalLayer.in_features
+            if originalLayer.bias is not None:
+                q.bias = nn.Parameter(originalLayer.bias.data.clone())
+            return q
         w_t = W.detach().cpu().to(torch.float16).t().contiguous()      # [Din, Dout]
         w_ref, packed, scale = layout.quantize_and_pack(w_t, group_size, given_scale, pad_out=q.pad_out)
         q.size_k, q.size_n = w_ref.shape
