@@ -114,3 +114,48 @@ def test_quantize_errors(gpu):
     with pytest.raises(RuntimeError):
         ops.w4a16_pack(torch.zeros(100, 128, dtype=torch.uint8, device=gpu),
                        torch.zeros(0, 128, dtype=torch.float16, device=gpu))
+
+
+def _full_layer(k, n, seed, dev):
+    rng = np.random.default_rng(seed)
+    q = rng.integers(0, 16, size=(k, n)).astype(np.int32)
+    s = rng.uniform(0.004, 0.02, size=(k // 128, n)).astype(np.float16)
+    packed = torch.from_numpy(O.pack_weights(q)).to(dev)
+    s_perm = torch.from_numpy(O.permute_scales(s, k, n, 128)).to(dev)
+    ws = torch.zeros((n // 64) * 16, dtype=torch.int32, device=dev)
+    return q, s, packed, s_perm, ws
+
+
+def test_slice_up_gate_proj(gpu):
+    """modeling_helpers.py:361-408 on the device: cut tensors equal unpack -> cut -> pack of the
+    oracle, and the cut layer computes the kept columns of the full layer."""
+    from uniql_amd import ops, slicing
+    hidden, inter, reduced = 512, 1024, 600          # kept width 600 -> padded to 768
+    q, s, packed, s_perm, ws = _full_layer(hidden, inter, 11, gpu)
+    w2, s2, ws2 = slicing.slice_w4a16_up_gate_proj(packed, s_perm, ws, hidden, inter, reduced, packed.shape)
+    s_cut = s[:, :768].copy()
+    s_cut[:, reduced:] = 0
+    assert np.array_equal(w2.cpu().numpy(), O.pack_weights(q[:, :768]))
+    assert np.array_equal(s2.cpu().numpy().view(np.uint16), O.permute_scales(s_cut, hidden, 768, 128).view(np.uint16))
+    assert ws2.numel() == (768 // 64) * 16
+    x = torch.randn(3, hidden, generator=torch.Generator().manual_seed(1)).half().to(gpu)
+    full = ops.w4a16o16_gemm(x, packed, s_perm, ws, 3, inter, hidden)
+    cut = ops.w4a16o16_gemm(x, w2, s2, ws2, 3, 768, hidden)
+    assert torch.equal(cut[:, :reduced], full[:, :reduced])
+    assert int(cut[:, reduced:].abs().max()) == 0
+
+
+def test_slice_down_proj(gpu):
+    """modeling_helpers.py:411-448 on the device: a prefix of whole K groups; the cut layer on
+    the first rows of the activations equals the full layer on activations zeroed past them."""
+    from uniql_amd import ops, slicing
+    hidden, inter, reduced = 512, 1024, 600          # kept rows 600 -> padded to 640 (5 groups)
+    q, s, packed, s_perm, ws = _full_layer(inter, hidden, 12, gpu)
+    w2, s2, ws2 = slicing.slice_w4a16_down_proj(packed, s_perm, ws, hidden, inter, reduced, packed.shape)
+    assert np.array_equal(w2.cpu().numpy(), O.pack_weights(q[:640]))
+    assert np.array_equal(s2.cpu().numpy().view(np.uint16), O.permute_scales(s[:5], 640, hidden, 128).view(np.uint16))
+    x = torch.randn(2, inter, generator=torch.Generator().manual_seed(2)).half().to(gpu)
+    x[:, reduced:] = 0
+    full = ops.w4a16o16_gemm(x, packed, s_perm, ws, 2, hidden, inter)
+    cut = ops.w4a16o16_gemm(x[:, :640].contiguous(), w2, s2, ws2, 2, hidden, 640)
+    assert torch.allclose(cut.float(), full.float(), atol=2e-3)
