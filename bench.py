@@ -13,7 +13,9 @@ from HBM, not from cache.  Steps are replayed as HIP graphs (one per weight copy
 so that launch overhead is the GPU's, not Python's.
 
 value = algorithmic bytes per step / time per step  (GB/s), algorithmic bytes of a
-linear = K N / 2 + (K/128) N 2 + M K 2 + M N 2.
+linear = K N / 2 + (K/128) N 2 + M K 2 + M N 2.  The same JSON line carries, under
+"prefill_gemm_m1024", the other half of the metric: the four linears at M = 1024 through
+the tiled MFMA kernel (TFLOP/s = 2 M K N / time, against 2.5 PFLOP/s dense fp16).
 
 --sweep additionally prints (stderr) and writes (gpurun_out/bench_sweep.json) the
 per-shape tables: decode M in {1,2,4,8}, prefill M in {256,1024,4096}, the pruned
@@ -40,7 +42,7 @@ LLC_BYTES = 256 << 20
 # HBM bytes per launch of the default workload (mean over the four linears) from two
 # rocprofv3 --pmc runs of this file, FETCH_SIZE and WRITE_SIZE, each scaled by the reading for a
 # 128 MiB elementwise copy (--pmc-calibrate): factors 2.000 and 1.000.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28838246
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28734222
 
 LLAMA_DECODE = [("qkv", 4096, 6144), ("o_proj", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
 PRUNED = [("q_pruned", 4096, 3584, 0), ("o_pruned", 3456, 4096, 0), ("gate_up_pruned", 4096, 24320, 0),
@@ -281,6 +283,25 @@ def main():
     }
     del layers
     torch.cuda.empty_cache()
+
+    # second half of the metric: the same four linears at M = 1024 through the tiled MFMA kernel
+    pm = 1024
+    per_shape, tot_flops, tot_sec = {}, 0.0, 0.0
+    for name, k, n in LLAMA_DECODE:
+        layer = Layer(name, k, n, pm, 2, dev, gen)
+        sec, _ = time_graphs(lambda i: layer.run(i), 2, 20, 4)
+        fl = linear_flops(pm, k, n)
+        per_shape[name] = {"us": round(sec * 1e6, 2), "tflops": round(fl / sec / 1e12, 1)}
+        tot_flops += fl
+        tot_sec += sec
+        del layer
+        torch.cuda.empty_cache()
+    result["prefill_gemm_m1024"] = {
+        "metric": "W4A16 prefill GEMM TFLOP/s at M=1024 (same four linears)", "value": round(tot_flops / tot_sec / 1e12, 1),
+        "unit": "TFLOP/s", "us_per_layer": round(tot_sec * 1e6, 2), "per_linear": per_shape,
+        "roofline": {"bound": "mfma", "achieved": round(tot_flops / tot_sec / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                     "unit": "TFLOP/s", "frac": round(tot_flops / tot_sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                     "kernel": "w4a16_tile_kernel<MT> (MT = 4, or 2 for the 6144-wide qkv)"}}
     if args.sweep:
         sweep(dev, gen, os.path.join(ROOT, "gpurun_out", "bench_sweep.json"))
     if not args.no_cpu:
