@@ -159,3 +159,55 @@ def test_slice_down_proj(gpu):
     full = ops.w4a16o16_gemm(x, packed, s_perm, ws, 2, hidden, inter)
     cut = ops.w4a16o16_gemm(x[:, :640].contiguous(), w2, s2, ws2, 2, hidden, 640)
     assert torch.allclose(cut.float(), full.float(), atol=2e-3)
+
+
+def test_slice_qk_and_v_proj(gpu):
+    """modeling_helpers.py:451-596 on the device: the cut layers compute exactly the kept
+    columns of the full layer (same codes, same scales, same K order), zeros in the padding."""
+    from uniql_amd import ops, slicing
+    hidden, nheads, head_dim, red = 512, 6, 128, 80           # 768 -> 480 columns, padded to 512
+    n_full = nheads * head_dim
+    q, s, packed, s_perm, ws = _full_layer(hidden, n_full, 21, gpu)
+    x = torch.randn(4, hidden, generator=torch.Generator().manual_seed(3)).half().to(gpu)
+    full = ops.w4a16o16_gemm(x, packed, s_perm, ws, 4, n_full, hidden)
+    bias = torch.arange(n_full, dtype=torch.float16, device=gpu)
+    # q/k: first red/2 columns of each rotary half of every head
+    w2, b2, s2, ws2 = slicing.slice_w4a16_qk_proj(packed, bias, s_perm, ws, hidden, nheads, head_dim, red, packed.shape)
+    cols = np.concatenate([h * head_dim + np.concatenate([np.arange(red // 2), head_dim // 2 + np.arange(red // 2)])
+                           for h in range(nheads)])
+    assert tuple(w2.shape) == (hidden // 16, 2 * 512) and ws2.numel() == (512 // 64) * 16
+    cut = ops.w4a16o16_gemm(x, w2, s2, ws2, 4, 512, hidden)
+    assert torch.equal(cut[:, :len(cols)], full[:, torch.from_numpy(cols).to(gpu)])
+    assert int(cut[:, len(cols):].abs().max()) == 0
+    assert torch.equal(b2, bias[torch.from_numpy(cols).to(gpu)])
+    assert np.array_equal(w2.cpu().numpy(), O.pack_weights(np.concatenate([q[:, cols], np.zeros((hidden, 32), np.int32)], 1)))
+    # v: the first `red` columns of every head
+    w3, s3, ws3 = slicing.slice_w4a16_v_proj(packed, s_perm, ws, hidden, nheads, head_dim, red, packed.shape)
+    vcols = np.concatenate([h * head_dim + np.arange(red) for h in range(nheads)])
+    cut = ops.w4a16o16_gemm(x, w3, s3, ws3, 4, 512, hidden)
+    assert torch.equal(cut[:, :len(vcols)], full[:, torch.from_numpy(vcols).to(gpu)])
+
+
+def test_slice_o_proj_requantises(gpu):
+    """modeling_helpers.py:600-656 on the device: dequantise, keep every head's first rows,
+    quantise again.  Equal to the oracle's quantiser on the oracle's dequantised weights, and
+    close to the full layer applied to activations that are zero in the dropped positions."""
+    from uniql_amd import ops, slicing
+    hidden, nheads, head_dim, red = 512, 6, 128, 80
+    k_full = nheads * head_dim
+    q, s, packed, s_perm, ws = _full_layer(k_full, hidden, 22, gpu)
+    w2, s2, ws2 = slicing.slice_w4a16_o_proj(packed, s_perm, ws, hidden, nheads, head_dim, red, packed.shape)
+    rows = np.concatenate([h * head_dim + np.arange(red) for h in range(nheads)])
+    w_deq = O.dequant_codes(q, s)                                           # fp16 [k, n]
+    _, o_packed, o_scale = O.w4a16_quantize(torch.from_numpy(w_deq[rows]), 128, None, 0)
+    assert tuple(w2.shape) == (512 // 16, 2 * hidden)                       # 480 rows -> 512
+    assert torch.equal(w2.cpu(), o_packed) and torch.equal(s2.cpu(), o_scale)
+    x = torch.randn(2, k_full, generator=torch.Generator().manual_seed(4)).half()
+    keep = torch.zeros(k_full, dtype=torch.bool)
+    keep[torch.from_numpy(rows)] = True
+    x_full = (x * keep).to(gpu)
+    x_cut = torch.nn.functional.pad(x[:, torch.from_numpy(rows)], (0, 512 - len(rows))).to(gpu).contiguous()
+    full = ops.w4a16o16_gemm(x_full, packed, s_perm, ws, 2, hidden, k_full)
+    cut = ops.w4a16o16_gemm(x_cut, w2, s2, ws2, 2, hidden, 512)
+    rel = (cut.float() - full.float()).abs().mean() / full.float().abs().mean()
+    assert rel < 0.1                                                        # re-quantisation noise only

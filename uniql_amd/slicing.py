@@ -63,3 +63,89 @@ def slice_w4a16_down_proj(weight, scale, workspace, hidden_size, intermediate_si
     new_weight = weight[:keep // 16].contiguous()
     new_scale = scale[:int(math.ceil(reduced_intermediate_size / 128))].contiguous()
     return new_weight, new_scale, workspace
+
+
+def _workspace_for(size_n: int, workspace):
+    return workspace[:(size_n // MIN_THREAD_N) * MAX_PARALLEL].contiguous()
+
+
+def _gather_columns(weight, scale, workspace, size_k, size_n, rows_real, cols: torch.Tensor, pad_n_new: int):
+    """Unpacks [size_k, size_n], keeps the real K rows and the columns `cols`, pads the rows back
+    to size_k with code 0 as the reference's torch.nn.functional.pad does, and packs with
+    pad_n_new padding columns (code 0, scale 0)."""
+    codes, scales = ops.w4a16_unpack(weight, scale, size_n, size_k)
+    cut = codes[:rows_real][:, cols]
+    if rows_real < size_k:
+        cut = torch.cat([cut, cut.new_zeros(size_k - rows_real, cut.shape[1])], dim=0)
+    new_weight, new_scale = ops.w4a16_pack(cut.contiguous(), scales[:, cols].contiguous(), pad_out=pad_n_new)
+    return new_weight, new_scale, _workspace_for(cols.numel() + pad_n_new, workspace)
+
+
+def _rope_half_columns(nheads, head_dim, reduced_head_dim, device):
+    """Per head, the first reduced_head_dim/2 columns of each rotary half
+    (modeling_helpers.py:481-486)."""
+    half, hd_half = head_dim // 2, reduced_head_dim // 2
+    d = torch.cat([torch.arange(hd_half, device=device), half + torch.arange(hd_half, device=device)])
+    return (torch.arange(nheads, device=device)[:, None] * head_dim + d[None, :]).reshape(-1)
+
+
+def _head_prefix(nheads, head_dim, reduced_head_dim, device):
+    d = torch.arange(reduced_head_dim, device=device)
+    return (torch.arange(nheads, device=device)[:, None] * head_dim + d[None, :]).reshape(-1)
+
+
+def slice_w4a16_qk_proj(weight, bias, scale, workspace, hidden_size, nheads, head_dim, reduced_head_dim,
+                        load_shape, num_bits=4, group_size=128):
+    """Query/key projection [hidden_size -> nheads * head_dim]: every head keeps the first
+    reduced_head_dim / 2 columns of each rotary half (modeling_helpers.py:451-530)."""
+    assert num_bits == 4, "Only support 4-bit quantization for now"
+    assert group_size == 128, "Only group_size 128 is supported on the device"
+    pad_k = _pad_to(hidden_size, group_size)
+    pad_n = _pad_to(nheads * head_dim, 256)
+    reduced_pad_n = _pad_to(nheads * reduced_head_dim, 256)
+    assert load_shape[0] == weight.shape[0], "hidden_size dimension mismatch"
+    cols = _rope_half_columns(nheads, head_dim, reduced_head_dim, weight.device)
+    new_weight, new_scale, new_workspace = _gather_columns(
+        weight, scale, workspace, hidden_size + pad_k, nheads * head_dim + pad_n, hidden_size, cols, reduced_pad_n)
+    new_bias = None if bias is None else bias[cols.to(bias.device)]
+    return new_weight, new_bias, new_scale, new_workspace
+
+
+def slice_w4a16_v_proj(weight, scale, workspace, hidden_size, nheads, head_dim, reduced_head_dim,
+                       load_shape, num_bits=4, group_size=128):
+    """Value projection: every head keeps its first reduced_head_dim columns
+    (modeling_helpers.py:533-596)."""
+    assert num_bits == 4, "Only support 4-bit quantization for now"
+    assert group_size == 128, "Only group_size 128 is supported on the device"
+    pad_k = _pad_to(hidden_size, group_size)
+    pad_n = _pad_to(nheads * head_dim, 256)
+    reduced_pad_n = _pad_to(nheads * reduced_head_dim, 256)
+    assert load_shape[0] == weight.shape[0], "hidden_size dimension mismatch"
+    cols = _head_prefix(nheads, head_dim, reduced_head_dim, weight.device)
+    return _gather_columns(weight, scale, workspace, hidden_size + pad_k, nheads * head_dim + pad_n, hidden_size,
+                           cols, reduced_pad_n)
+
+
+def slice_w4a16_o_proj(weight, scale, workspace, hidden_size, nheads, head_dim, reduced_head_dim,
+                       load_shape, num_bits=4, group_size=128):
+    """Output projection [nheads * head_dim -> hidden_size]: the kept input rows do not line up
+    with the groups of 128 any more, so the reference dequantises, keeps every head's first
+    reduced_head_dim rows and quantises again (modeling_helpers.py:600-656); the same here with
+    the device kernels (bit-exact fp16 weights out of uniql_w4a16_dequant, uniql_w4a16_quantize)."""
+    assert num_bits == 4, "Only support 4-bit quantization for now"
+    assert group_size == 128, "Only group_size 128 is supported on the device"
+    pad_k = _pad_to(nheads * head_dim, group_size)
+    pad_n = _pad_to(hidden_size, 256)
+    assert load_shape[1] == weight.shape[1], "hidden_size dimension mismatch"
+    size_k, size_n = nheads * head_dim + pad_k, hidden_size + pad_n
+    w_full = ops.w4a16_dequant(weight, scale, size_n, size_k)              # fp16 (code - 8) * scale, [k, n]
+    rows = _head_prefix(nheads, head_dim, reduced_head_dim, weight.device)
+    kept = w_full[rows][:, :hidden_size]                                  # [nheads * reduced_head_dim, hidden]
+    new_weight, new_scale = ops.w4a16_quantize(kept.t().contiguous(), None, pad_out=pad_n)
+    return new_weight, new_scale, workspace
+
+
+def slice_indices(indices, head_dim, reduced_head_dim):
+    """modeling_helpers.py:659-663."""
+    half, hd_half = head_dim // 2, reduced_head_dim // 2
+    return torch.cat([indices[:, :hd_half], indices[:, half:half + hd_half]], dim=-1).to(torch.uint8)
