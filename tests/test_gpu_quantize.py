@@ -211,3 +211,42 @@ def test_slice_o_proj_requantises(gpu):
     cut = ops.w4a16o16_gemm(x_cut, w2, s2, ws2, 2, hidden, 512)
     rel = (cut.float() - full.float()).abs().mean() / full.float().abs().mean()
     assert rel < 0.1                                                        # re-quantisation noise only
+
+
+def test_slice_mamba_in_and_out_proj(gpu):
+    """modeling_helpers.py:665-867 on the device, on a small Mamba2-shaped block."""
+    from uniql_amd import ops, slicing
+    hidden, n_groups, num_heads, inter, state = 256, 2, 8, 512, 64
+    load_inter, load_state = 384, 48                      # head_dim 64 -> 48, states 64 -> 48
+    proj = 2 * inter + 2 * n_groups * state + num_heads   # 1288 -> padded to 1536
+    n_full = proj + (-proj) % 256
+    q, s, packed, s_perm, ws = _full_layer(hidden, n_full, 31, gpu)
+    w2, s2, ws2 = slicing.slice_w4a16_in_proj(packed, s_perm, ws, hidden, n_groups, num_heads, inter, state,
+                                              load_inter, load_state, packed.shape)
+    heads = np.concatenate([h * 64 + np.arange(48) for h in range(num_heads)])
+    states = np.concatenate([g * state + np.arange(load_state) for g in range(n_groups)])
+    cols = np.concatenate([heads, inter + heads, 2 * inter + states, 2 * inter + n_groups * state + states,
+                           np.arange(2 * inter + 2 * n_groups * state, proj)])
+    red = 2 * load_inter + 2 * n_groups * load_state + num_heads
+    assert len(cols) == red
+    n_cut = red + (-red) % 256
+    assert tuple(w2.shape) == (hidden // 16, 2 * n_cut)
+    x = torch.randn(3, hidden, generator=torch.Generator().manual_seed(6)).half().to(gpu)
+    full = ops.w4a16o16_gemm(x, packed, s_perm, ws, 3, n_full, hidden)
+    cut = ops.w4a16o16_gemm(x, w2, s2, ws2, 3, n_cut, hidden)
+    assert torch.equal(cut[:, :red], full[:, torch.from_numpy(cols).to(gpu)])
+    assert int(cut[:, red:].abs().max()) == 0
+    # out_proj: dequantise, keep head prefixes, quantise again == the oracle's quantiser on the kept rows
+    q, s, packed, s_perm, ws = _full_layer(inter, hidden, 32, gpu)
+    w3, s3, _ = slicing.slice_w4a16_out_proj(packed, s_perm, ws, hidden, n_groups, num_heads, inter, load_inter,
+                                             packed.shape)
+    _, o_packed, o_scale = O.w4a16_quantize(torch.from_numpy(O.dequant_codes(q, s)[heads]), 128, None, 0)
+    assert torch.equal(w3.cpu(), o_packed) and torch.equal(s3.cpu(), o_scale)
+    # the convolution and norm cuts follow the same index lists
+    conv_w = torch.arange((inter + 2 * n_groups * state) * 4, dtype=torch.float32, device=gpu).reshape(-1, 1, 4)
+    conv_b = torch.arange(inter + 2 * n_groups * state, dtype=torch.float32, device=gpu)
+    cw, cb = slicing.slice_conv1d(conv_w, conv_b, n_groups, num_heads, inter, state, load_inter, load_state)
+    want = np.concatenate([heads, inter + states, inter + n_groups * state + states])
+    assert np.array_equal(cb.cpu().numpy(), want.astype(np.float32)) and cw.shape[0] == len(want)
+    nw = slicing.slice_norm(torch.arange(inter, dtype=torch.float32, device=gpu), n_groups, num_heads, inter, load_inter)
+    assert np.array_equal(nw.cpu().numpy(), heads.astype(np.float32))

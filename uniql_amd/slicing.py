@@ -149,3 +149,80 @@ def slice_indices(indices, head_dim, reduced_head_dim):
     """modeling_helpers.py:659-663."""
     half, hd_half = head_dim // 2, reduced_head_dim // 2
     return torch.cat([indices[:, :hd_half], indices[:, half:half + hd_half]], dim=-1).to(torch.uint8)
+
+
+def get_topk_head_indices(n_groups, num_heads, head_dim, topk_head_dim, device=None):
+    """First topk_head_dim channels of every head (modeling_helpers.py:124-130; the grouping of
+    heads does not change their order)."""
+    return _head_prefix(num_heads, head_dim, topk_head_dim, device)
+
+
+def get_topk_ssm_state_indices(n_groups, ssm_state_size, topk_ssm_state, device=None):
+    """First topk_ssm_state states of every group (modeling_helpers.py:132-137)."""
+    return _head_prefix(n_groups, ssm_state_size, topk_ssm_state, device)
+
+
+def slice_w4a16_in_proj(weight, scale, workspace, hidden_size, n_groups, num_heads, intermediate_size,
+                        ssm_state_size, load_intermediate_size, load_ssm_state_size, load_shape,
+                        num_bits=4, group_size=128):
+    """Mamba2 input projection [hidden -> z | x | B | C | dt]: z and x keep the first channels
+    of every head, B and C the first states of every group, dt stays
+    (modeling_helpers.py:665-757)."""
+    assert num_bits == 4, "Only support 4-bit quantization for now"
+    assert group_size == 128, "Only group_size 128 is supported on the device"
+    projection_size = 2 * intermediate_size + 2 * n_groups * ssm_state_size + num_heads
+    reduced_projection_size = 2 * load_intermediate_size + 2 * n_groups * load_ssm_state_size + num_heads
+    pad_k = _pad_to(hidden_size, group_size)
+    pad_n = _pad_to(projection_size, 256)
+    reduced_pad_n = _pad_to(reduced_projection_size, 256)
+    assert load_shape[0] == weight.shape[0], "hidden_size dimension mismatch"
+    dev = weight.device
+    heads = get_topk_head_indices(n_groups, num_heads, intermediate_size // num_heads,
+                                  load_intermediate_size // num_heads, dev)
+    states = get_topk_ssm_state_indices(n_groups, ssm_state_size, load_ssm_state_size, dev)
+    x_start = intermediate_size
+    b_start = x_start + intermediate_size
+    c_start = b_start + n_groups * ssm_state_size
+    dt_start = c_start + n_groups * ssm_state_size
+    cols = torch.cat([heads, x_start + heads, b_start + states, c_start + states,
+                      torch.arange(dt_start, projection_size, device=dev)])
+    return _gather_columns(weight, scale, workspace, hidden_size + pad_k, projection_size + pad_n, hidden_size,
+                           cols, reduced_pad_n)
+
+
+def slice_w4a16_out_proj(weight, scale, workspace, hidden_size, n_groups, num_heads, intermediate_size,
+                         load_intermediate_size, load_shape, num_bits=4, group_size=128):
+    """Mamba2 output projection [intermediate -> hidden]: dequantise, keep the first channels of
+    every head, quantise again (modeling_helpers.py:809-867)."""
+    assert num_bits == 4, "Only support 4-bit quantization for now"
+    assert group_size == 128, "Only group_size 128 is supported on the device"
+    pad_k = _pad_to(intermediate_size, group_size)
+    pad_n = _pad_to(hidden_size, 256)
+    assert load_shape[1] == weight.shape[1], "hidden_size dimension mismatch"
+    w_full = ops.w4a16_dequant(weight, scale, hidden_size + pad_n, intermediate_size + pad_k)
+    rows = get_topk_head_indices(n_groups, num_heads, intermediate_size // num_heads,
+                                 load_intermediate_size // num_heads, weight.device)
+    kept = w_full[rows][:, :hidden_size]
+    new_weight, new_scale = ops.w4a16_quantize(kept.t().contiguous(), None, pad_out=pad_n)
+    return new_weight, new_scale, workspace
+
+
+def slice_conv1d(weight, bias, n_groups, num_heads, intermediate_size, ssm_state_size,
+                 load_intermediate_size, load_ssm_state_size):
+    """The matching cut of Mamba2's depthwise convolution over x | B | C
+    (modeling_helpers.py:760-790)."""
+    dev = weight.device
+    heads = get_topk_head_indices(n_groups, num_heads, intermediate_size // num_heads,
+                                  load_intermediate_size // num_heads, dev)
+    states = get_topk_ssm_state_indices(n_groups, ssm_state_size, load_ssm_state_size, dev)
+    b_start = intermediate_size
+    c_start = b_start + n_groups * ssm_state_size
+    idx = torch.cat([heads, b_start + states, c_start + states])
+    return weight[idx].contiguous(), bias[idx].contiguous()
+
+
+def slice_norm(weight, n_groups, num_heads, intermediate_size, load_intermediate_size):
+    """modeling_helpers.py:793-800."""
+    idx = get_topk_head_indices(n_groups, num_heads, intermediate_size // num_heads,
+                                load_intermediate_size // num_heads, weight.device)
+    return weight[idx].contiguous()
