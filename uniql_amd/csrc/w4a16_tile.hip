@@ -26,7 +26,8 @@
 //     sg ^ (r % 16);
 //   * per wave, its two packed rows of the strip (2 x 1 KiB): piece (c8, ch, kq) at position
 //     c8 + 8 ch + 16 kq, so a half-wave's 8-byte reads sweep all 64 banks;
-//   * per wave, the 256 bytes of scales of the strip (four copies, one per quarter-wave).
+//   * the 256 bytes of scales of the strip (four copies, one per quarter-wave; every wave
+//     writes all of them with the same values).
 // vmcnt is counted by hand: every stage issues exactly kStageOps LDS-DMA operations per
 // wave and nothing else uses the counter inside the loop.
 //
@@ -69,7 +70,7 @@ struct TileLds {
     static constexpr int kRows = 32 * MT;
     static constexpr int kXDwords = kRows * 64;        // X tile
     static constexpr int kBDwords = 4 * 2 * 256;       // 4 waves x 2 packed rows x 1 KiB
-    static constexpr int kSDwords = 4 * 256;           // 4 waves x 4 copies of the strip's 256 bytes of scales
+    static constexpr int kSDwords = 256;               // 4 copies of the strip's 256 bytes of scales
     static constexpr int kStageDwords = kXDwords + kBDwords + kSDwords;
     static constexpr size_t kRingBytes = (size_t)kRing * kStageDwords * 4;
     static constexpr size_t kRedBytes = (size_t)4 * 32 * 132 * 4;  // 4 waves x one 32-row M tile, fp32, padded rows
@@ -174,9 +175,10 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
             __builtin_amdgcn_global_load_lds((gptr_t)(rowp + piece_off), (lptr_t)bbuf, 16, 0, 0);
         } else {
             // scales of the group (row 0 in per-column mode, unused then)
-            // all 64 lanes take part (a predicated load would split the loop body into several
-            // scheduling regions): the four quarter-waves fetch the same 256 bytes
-            uint32_t* sbuf = stage + L::kXDwords + L::kBDwords + w * 256;
+            // all 64 lanes of all four waves take part (a predicated load would split the loop
+            // body into several scheduling regions): every quarter-wave fetches the same 256
+            // bytes, and the four waves write the same values to the same place
+            uint32_t* sbuf = stage + L::kXDwords + L::kBDwords;
             const half_t* ssrc = strip_s + (size_t)g * scale_row_stride;
             __builtin_amdgcn_global_load_lds((gptr_t)(ssrc + 8 * dslot), (lptr_t)sbuf, 16, 0, 0);
         }
@@ -207,7 +209,7 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     auto read_words = [&](int set, int ring) __attribute__((always_inline)) {
         const uint32_t* stage = lds + ring * L::kStageDwords;
         const uint32_t* bbuf = stage + L::kXDwords + w * 512;
-        const u32x2 sc_lds = *reinterpret_cast<const u32x2*>(stage + L::kXDwords + L::kBDwords + w * 256 + soff);
+        const u32x2 sc_lds = *reinterpret_cast<const u32x2*>(stage + L::kXDwords + L::kBDwords + soff);
         scv[set] = a.per_column ? sc_fixed : sc_lds;
 #pragma unroll
         for (int t = 0; t < 2; ++t) {
