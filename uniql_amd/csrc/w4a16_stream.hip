@@ -75,9 +75,10 @@ __device__ __forceinline__ void store_out(const StreamArgs& a, int m, int n, flo
 // (1, 2, 4, 8, 16): it fixes NV, how many of the four output rows of a lane's accumulator
 // quad are real, and XQ, how many quads of activation rows are loaded and staged.  WAVES: wavefronts
 // per workgroup (4, 8 or 16); with 16 a workgroup can cover all of K for shapes with many
-// strips, which removes the exchange of partial sums between workgroups.  PF: prefetch the
-// next group's weights into a second register set while the current one is consumed.
-template <int MT, int RC, bool HAD, int WAVES, bool PF>
+// strips, which removes the exchange of partial sums between workgroups.  A wave keeps one
+// group's weights in registers at a time: a second register set for the next group costs more
+// in occupancy than it hides in latency, the other waves of the SIMD do that.
+template <int MT, int RC, bool HAD, int WAVES>
 __global__ __launch_bounds__(64 * WAVES, (MT == 1 ? (WAVES == 16 ? 4 : 3) : (MT == 2 ? 2 : 1)))
 void w4a16_stream_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
@@ -168,10 +169,8 @@ void w4a16_stream_kernel(const StreamArgs a) {
         for (int rr = 0; rr < 2 * RPW; ++rr) wq[rr] = __builtin_nontemporal_load(rowp + (size_t)rr * N4 + piece_off);
     };
 
-    if (PF && g_begin < g_end) issue_loads(g_begin);
-
     for (int g = g_begin; g < g_end; ++g) {  // wave-uniform trip count
-        if (!PF) issue_loads(g);
+        issue_loads(g);
         // ---- rotate (optionally) and stage the activations in LDS ------------------
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
@@ -219,17 +218,13 @@ void w4a16_stream_kernel(const StreamArgs a) {
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        u32x4 cur[2 * RPW];
-#pragma unroll
-        for (int rr = 0; rr < 2 * RPW; ++rr) cur[rr] = wq[rr];
+        const u32x4 (&cur)[2 * RPW] = wq;
         const u32x4 sc_cur = sc;
-        // all activation rows this group needs, fetched from LDS before the next group's
-        // loads overwrite the staging registers
         h8 xa[RPW][MT];
         f4 zp[MT];  // minus 8 * row sums for this lane's four output rows: the first MFMA's C operand
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            if (PF || WAVES != 16) {
+            if (WAVES != 16) {
 #pragma unroll
                 for (int rp = 0; rp < RPW; ++rp)
                     xa[rp][mt] = __builtin_bit_cast(
@@ -242,8 +237,6 @@ void w4a16_stream_kernel(const StreamArgs a) {
                 zp[mt][v] = (v >= NV) ? 0.f : -sums[0];
             }
         }
-        if (PF && g + 1 < g_end) issue_loads(g + 1);
-
         // two passes over the columns (word pairs j) keep the group's raw dot products in
         // sixteen registers; the scale of output column jb of this lane is half jb of the
         // 16-byte scale load
@@ -254,7 +247,7 @@ void w4a16_stream_kernel(const StreamArgs a) {
             for (int rp = 0; rp < RPW; ++rp) {
                 // 16-wave workgroups live on 128 registers: they re-read the activations from
                 // LDS in each pass instead of holding all four row pairs
-                if (!PF && WAVES == 16) {
+                if (WAVES == 16) {
 #pragma unroll
                     for (int mt = 0; mt < MT; ++mt)
                         xa[rp][mt] = __builtin_bit_cast(
@@ -368,34 +361,37 @@ struct StreamPlan {
     int waves;  // 4, 8 or 16
     int upw;    // groups per wave
     int splits;
-    bool prefetch;
 };
 
-// Heuristic (from sweeps over waves x groups per wave on the Llama shapes): shapes with enough
-// strips to occupy the chip on their own let one workgroup own a whole strip, so no partial
-// sums are exchanged: 8 waves without the second register set (two workgroups per compute
-// unit) for one or two rows, 16 waves for more rows; otherwise K is split over workgroups of
-// 4 waves, or of 8 when that still leaves fewer than three waves per SIMD.
+// Heuristic (from sweeps over waves x groups per wave on the Llama shapes):
+//   * enough strips to occupy the chip on their own (>= 192): one workgroup of 8 waves owns a
+//     whole strip, so no partial sums are exchanged between workgroups;
+//   * otherwise K is split over workgroups.  One or two rows: 4 waves (8 when that still leaves
+//     fewer than three waves per SIMD), about 1024 workgroups at most.  More rows: every split
+//     costs a 64-bit atomic per output element, so 8 waves and at most about 256 workgroups.
 static StreamPlan stream_plan(int m, int n, int k, int upw_override, int waves_override) {
     const int nstrips = n / 128, G = k / 128;
+    const int64_t units = (int64_t)nstrips * G;
     StreamPlan p;
-    p.waves = 4;
-    p.prefetch = true;
     const bool whole_strip = m <= 16 && nstrips >= 192 && G >= 16 && G <= 64;
-    if (waves_override) p.waves = waves_override;
-    else if (whole_strip) p.waves = m <= 2 ? 8 : 16;
-    else if (m <= 2 && (int64_t)nstrips * G >= 1536 && (int64_t)nstrips * G < 3072) p.waves = 8;
+    int max_wgs = 1024;
+    if (waves_override) {
+        p.waves = waves_override;
+    } else if (whole_strip) {
+        p.waves = 8;
+    } else if (m <= 2) {
+        p.waves = (units >= 1536 && units < 3072) ? 8 : 4;
+    } else {
+        p.waves = (m <= 16 && units >= 1536) ? 8 : 4;
+        max_wgs = 256;
+    }
     if (upw_override > 0) {
         p.upw = upw_override;
     } else if (whole_strip && !waves_override) {
         p.upw = ceil_div(G, p.waves);
-        p.prefetch = false;
-    } else if (p.waves == 16) {
-        p.upw = ceil_div(G, 16);
-        if (p.upw > 8) p.upw = 8;
     } else {
         p.upw = 1;
-        while (p.upw < 8 && (int64_t)nstrips * ceil_div(G, p.waves * p.upw) > 1024) p.upw *= 2;
+        while (p.upw < 8 && (int64_t)nstrips * ceil_div(G, p.waves * p.upw) > max_wgs) p.upw *= 2;
     }
     p.splits = ceil_div(G, p.waves * p.upw);
     while (p.splits > 255) {  // the contribution count has 8 bits
@@ -413,12 +409,12 @@ size_t stream_accum_bytes(int m, int n, int k) {
     return (size_t)mrows * n * sizeof(unsigned long long);
 }
 
-template <int MT, int RC, bool HAD, int WAVES, bool PF>
+template <int MT, int RC, bool HAD, int WAVES>
 static hipError_t launch_one(const StreamArgs& a, hipStream_t stream) {
     const size_t stage = (size_t)WAVES * a.xrows * kXsStride * 4;
     const size_t red = a.xrows <= 4 ? (size_t)WAVES * 4 * 128 * 4 : (size_t)4 * 16 * 128 * 4;
     const size_t shmem = stage + red;
-    auto kern = &w4a16_stream_kernel<MT, RC, HAD, WAVES, PF>;
+    auto kern = &w4a16_stream_kernel<MT, RC, HAD, WAVES>;
     if (shmem > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -430,29 +426,28 @@ static hipError_t launch_one(const StreamArgs& a, hipStream_t stream) {
 }
 
 template <int MT, int RC, bool HAD>
-static hipError_t launch_waves(const StreamArgs& a, int waves, bool pf, hipStream_t stream) {
+static hipError_t launch_waves(const StreamArgs& a, int waves, hipStream_t stream) {
     if constexpr (MT == 1) {
-        if (waves == 16) return launch_one<MT, RC, HAD, 16, false>(a, stream);  // 128-register budget: no second weight set
-        if (waves == 8)
-            return pf ? launch_one<MT, RC, HAD, 8, true>(a, stream) : launch_one<MT, RC, HAD, 8, false>(a, stream);
+        if (waves == 16) return launch_one<MT, RC, HAD, 16>(a, stream);
+        if (waves == 8) return launch_one<MT, RC, HAD, 8>(a, stream);
     }
-    return pf ? launch_one<MT, RC, HAD, 4, true>(a, stream) : launch_one<MT, RC, HAD, 4, false>(a, stream);
+    return launch_one<MT, RC, HAD, 4>(a, stream);
 }
 
 template <bool HAD>
-static hipError_t launch_rows(const StreamArgs& a, int mt, int waves, bool pf, hipStream_t stream) {
-    if (mt == 4) return launch_waves<4, 16, HAD>(a, waves, pf, stream);
-    if (mt == 2) return launch_waves<2, 16, HAD>(a, waves, pf, stream);
-    if (a.M == 1) return launch_waves<1, 1, HAD>(a, waves, pf, stream);
-    if (a.M == 2) return launch_waves<1, 2, HAD>(a, waves, pf, stream);
-    if (a.M <= 4) return launch_waves<1, 4, HAD>(a, waves, pf, stream);
-    if (a.M <= 8) return launch_waves<1, 8, HAD>(a, waves, pf, stream);
-    return launch_waves<1, 16, HAD>(a, waves, pf, stream);
+static hipError_t launch_rows(const StreamArgs& a, int mt, int waves, hipStream_t stream) {
+    if (mt == 4) return launch_waves<4, 16, HAD>(a, waves, stream);
+    if (mt == 2) return launch_waves<2, 16, HAD>(a, waves, stream);
+    if (a.M == 1) return launch_waves<1, 1, HAD>(a, waves, stream);
+    if (a.M == 2) return launch_waves<1, 2, HAD>(a, waves, stream);
+    if (a.M <= 4) return launch_waves<1, 4, HAD>(a, waves, stream);
+    if (a.M <= 8) return launch_waves<1, 8, HAD>(a, waves, stream);
+    return launch_waves<1, 16, HAD>(a, waves, stream);
 }
 
 // Rows are processed in slabs of at most 64; every slab re-streams the weights.
-// tune: bits 0..7 groups per wave, bits 8..12 waves per workgroup (4/8/16), bit 13 no prefetch;
-// zero fields mean "choose".
+// tune: bits 0..7 groups per wave, bits 8..12 waves per workgroup (4/8/16); zero fields mean
+// "choose".
 int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, void* accum, int m, int n,
                   int k, int groups, bool had128, float had_scale, bool out_f32, unsigned tune,
                   hipStream_t stream) {
@@ -480,9 +475,8 @@ int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void
         a.xrows = mt == 1 ? ((mm + 3) / 4) * 4 : mt * 16;
         a.X = reinterpret_cast<const half_t*>(A) + (size_t)m0 * lda;
         a.D = reinterpret_cast<char*>(D) + (size_t)m0 * n * out_elt;
-        const bool pf = !(tune & 0x2000u) && plan.prefetch && plan.upw > 1 && plan.waves != 16;
-        const hipError_t e = had128 ? launch_rows<true>(a, mt, plan.waves, pf, stream)
-                                    : launch_rows<false>(a, mt, plan.waves, pf, stream);
+        const hipError_t e = had128 ? launch_rows<true>(a, mt, plan.waves, stream)
+                                    : launch_rows<false>(a, mt, plan.waves, stream);
         if (e != hipSuccess) return UNIQL_E_LAUNCH;
     }
     return UNIQL_OK;
