@@ -39,7 +39,7 @@ enum {
     UNIQL_F_FORCE_TILED = 1 << 2,  /* use the tiled MFMA kernel (default for m > 16) whatever m is */
     UNIQL_F_TRANSPOSE_OUT = 1 << 3 /* reference's output_transpose; rejected with UNIQL_E_UNSUPPORTED */
     /* tuning hooks, 0 = choose.  Streaming kernel: bits 8..15 K-groups per wavefront,
-       bits 16..20 wavefronts per workgroup (4, 8 or 16).
+       bits 16..20 wavefronts per workgroup (4 or 8).
        Tiled kernel: bits 8..15 number of K splits over workgroups, bits 16..19 row tiles of 32
        per workgroup (1, 2 or 4). */
 };

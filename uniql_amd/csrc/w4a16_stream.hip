@@ -73,13 +73,13 @@ __device__ __forceinline__ void store_out(const StreamArgs& a, int m, int n, flo
 
 // MT: 16-row tiles of M per workgroup.  RC: row class, an upper bound of M for MT = 1
 // (1, 2, 4, 8, 16): it fixes NV, how many of the four output rows of a lane's accumulator
-// quad are real, and XQ, how many quads of activation rows are loaded and staged.  WAVES: wavefronts
-// per workgroup (4, 8 or 16); with 16 a workgroup can cover all of K for shapes with many
-// strips, which removes the exchange of partial sums between workgroups.  A wave keeps one
+// quad are real, and XQ, how many quads of activation rows are loaded and staged.  WAVES:
+// wavefronts per workgroup (4 or 8); with 8 a workgroup can cover all of K for shapes with
+// many strips, which removes the exchange of partial sums between workgroups.  A wave keeps one
 // group's weights in registers at a time: a second register set for the next group costs more
 // in occupancy than it hides in latency, the other waves of the SIMD do that.
 template <int MT, int RC, bool HAD, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, (MT == 1 ? (WAVES == 16 ? 4 : 3) : (MT == 2 ? 2 : 1)))
+__global__ __launch_bounds__(64 * WAVES, (MT == 1 ? 3 : (MT == 2 ? 2 : 1)))
 void w4a16_stream_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     constexpr int NV = RC < 4 ? RC : 4;
@@ -224,12 +224,9 @@ void w4a16_stream_kernel(const StreamArgs a) {
         f4 zp[MT];  // minus 8 * row sums for this lane's four output rows: the first MFMA's C operand
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
-            if (WAVES != 16) {
 #pragma unroll
-                for (int rp = 0; rp < RPW; ++rp)
-                    xa[rp][mt] = __builtin_bit_cast(
-                        h8, *reinterpret_cast<const u32x4*>(xs + xrow_of[mt] + 16 * rp));
-            }
+            for (int rp = 0; rp < RPW; ++rp)
+                xa[rp][mt] = __builtin_bit_cast(h8, *reinterpret_cast<const u32x4*>(xs + xrow_of[mt] + 16 * rp));
 #pragma unroll
             for (int v = 0; v < 4; ++v) {
                 const int r = mt * 16 + 4 * kq + v;
@@ -245,14 +242,6 @@ void w4a16_stream_kernel(const StreamArgs a) {
             f4 dot[MT][4];
 #pragma unroll
             for (int rp = 0; rp < RPW; ++rp) {
-                // 16-wave workgroups live on 128 registers: they re-read the activations from
-                // LDS in each pass instead of holding all four row pairs
-                if (WAVES == 16) {
-#pragma unroll
-                    for (int mt = 0; mt < MT; ++mt)
-                        xa[rp][mt] = __builtin_bit_cast(
-                            h8, *reinterpret_cast<const u32x4*>(xs + xrow_of[mt] + 16 * rp));
-                }
 #pragma unroll
                 for (int jl = 0; jl < 2; ++jl) {
                     const int j = 2 * jh + jl;
@@ -358,7 +347,7 @@ void w4a16_stream_kernel(const StreamArgs a) {
 static inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
 struct StreamPlan {
-    int waves;  // 4, 8 or 16
+    int waves;  // 4 or 8
     int upw;    // groups per wave
     int splits;
 };
@@ -428,7 +417,6 @@ static hipError_t launch_one(const StreamArgs& a, hipStream_t stream) {
 template <int MT, int RC, bool HAD>
 static hipError_t launch_waves(const StreamArgs& a, int waves, hipStream_t stream) {
     if constexpr (MT == 1) {
-        if (waves == 16) return launch_one<MT, RC, HAD, 16>(a, stream);
         if (waves == 8) return launch_one<MT, RC, HAD, 8>(a, stream);
     }
     return launch_one<MT, RC, HAD, 4>(a, stream);
@@ -446,7 +434,7 @@ static hipError_t launch_rows(const StreamArgs& a, int mt, int waves, hipStream_
 }
 
 // Rows are processed in slabs of at most 64; every slab re-streams the weights.
-// tune: bits 0..7 groups per wave, bits 8..12 waves per workgroup (4/8/16); zero fields mean
+// tune: bits 0..7 groups per wave, bits 8..12 waves per workgroup (4 or 8); zero fields mean
 // "choose".
 int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, void* accum, int m, int n,
                   int k, int groups, bool had128, float had_scale, bool out_f32, unsigned tune,
@@ -463,7 +451,7 @@ int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void
     a.out_f32 = out_f32 ? 1 : 0;
     a.had_scale = had_scale;
     int waves_override = (int)((tune >> 8) & 0x1fu);
-    if (waves_override != 4 && waves_override != 8 && waves_override != 16) waves_override = 0;
+    if (waves_override != 4 && waves_override != 8) waves_override = 0;
     const size_t out_elt = out_f32 ? 4 : 2;
     for (int m0 = 0; m0 < m; m0 += 64) {
         const int mm = (m - m0) < 64 ? (m - m0) : 64;
