@@ -222,3 +222,50 @@ def test_errors(gpu):
         ops.w4a16o16_gemm(x.cpu(), b, s, ws, 1, 256, 256)                 # no CPU path
     y = ops.w4a16o16_gemm(x[:0], b, s, ws, 0, 256, 256)
     assert tuple(y.shape) == (0, 256)
+
+
+# ------------------------------------------------------------------ streams and graphs
+def test_side_stream_and_graph_replay(gpu):
+    """Every entry point only enqueues kernels on the stream it is given: the calls can be
+    captured in a HIP graph and replayed, with eager work between the replays, and each replay
+    gives the eager result again (the accumulator words return to zero after every call)."""
+    from uniql_amd import ops
+    problems = [make_linear_problem(1, 4096, 512, seed=301),      # streaming kernel, K split with atomics
+                make_linear_problem(40, 1408, 256, seed=302),     # tiled kernel
+                make_linear_problem(3, 1536, 256, seed=303)]      # streaming kernel with the fused rotation
+    dev_in = [to_gpu(p, gpu) for p in problems]
+    ws = [workspace_for(p["n"], gpu) for p in problems]
+
+    def run_all():
+        outs = []
+        for i, (p, (x, b, s)) in enumerate(zip(problems, dev_in)):
+            kw = dict(had_block=128, had_scale=128 ** -0.5) if i == 2 else {}
+            outs.append(ops.w4a16_gemm_ex(x, b, s, ws[i], p["m"], p["n"], p["k"], **kw))
+        return outs
+
+    eager = [y.clone() for y in run_all()]
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        on_side = [y.clone() for y in run_all()]                  # also sizes the side stream's accumulators
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    for a, b in zip(eager, on_side):
+        assert torch.equal(a, b)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = run_all()
+    for rep in range(3):
+        for y in captured:
+            y.fill_(float("nan"))
+        graph.replay()
+        torch.cuda.synchronize()
+        for a, b in zip(eager, captured):
+            assert torch.equal(a, b), f"replay {rep}"
+        # eager work between the replays, on the same buffers' neighbours
+        again = run_all()
+        torch.cuda.synchronize()
+        for a, b in zip(eager, again):
+            assert torch.equal(a, b)
+    for buf in ops._accum_cache.values():
+        assert int(buf.count_nonzero()) == 0
