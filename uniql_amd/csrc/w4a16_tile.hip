@@ -441,24 +441,29 @@ size_t tile_accum_bytes(int m, int n, int k) {
     return tile_plan(m, n, k, 0).splits > 1 ? (size_t)m * n * sizeof(unsigned long long) : 0;
 }
 
-// Measured on MI355X (K groups of 128, one 32-row tile = "row tile"):
-//   * a workgroup of MT row tiles spends about 0.7 / 1.1 / 1.4 us per K group (MT = 1 / 2 / 4)
-//     when it has a compute unit to itself; per row tile the larger ones are the more
-//     efficient (they expand every weight once for MT row tiles), and two MT = 2 workgroups
-//     sharing a compute unit match one MT = 4 workgroup;
+// Measured on MI355X, in units of the time one MT = 4 workgroup takes for its K loop when every
+// compute unit has one ("a round"):
+//   * MT = 4: one workgroup per compute unit, every started round of 256 costs 1;
+//   * MT = 2: two workgroups share a compute unit; a full round of 512 costs 1.08 (every weight
+//     is expanded twice per 128 rows), a last round of at most 256 costs 0.85;
+//   * MT = 1: up to four share a compute unit: 0.62 for at most 256 workgroups, 0.88 for at most
+//     512, 1.62 per started round of 1024;
 //   * the exchange of partial sums costs one 64-bit atomic per output element and K split,
 //     about 150 G atomics/s for the chip.
-// So: the largest MT that still yields about one workgroup per compute unit; MT = 2 instead of
-// 4 when the MT = 4 grid would leave the last round of 256 workgroups mostly empty; K splits
-// only for MT = 1 grids that cannot fill the chip, and only while the atomics cost less than
-// the K loop they save.
+// So: the MT with the cheapest grid; K splits only for MT = 1 grids that cannot fill the chip,
+// and only while the atomics cost less than the K loop they save.
 static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_override) {
     TilePlan p;
     const int strips = n / 128, G = k / 128;
     const int64_t t4 = (int64_t)strips * ceil_div_i(m, 128), t2 = (int64_t)strips * ceil_div_i(m, 64);
-    if (t4 >= 256) p.mtiles = (t4 % 256 == 0 || t4 >= 1024) ? 4 : 2;
-    else if (t2 >= 200) p.mtiles = 2;
-    else p.mtiles = 1;
+    const int64_t t1 = (int64_t)strips * ceil_div_i(m, 32);
+    const double cost4 = (double)((t4 + 255) / 256);
+    const int64_t rem2 = t2 % 512;
+    const double cost2 = 1.08 * (double)(t2 / 512) + (rem2 == 0 ? 0.0 : (rem2 <= 256 ? 0.85 : 1.08));
+    const double cost1 = t1 <= 256 ? 0.62 : (t1 <= 512 ? 0.88 : 1.62 * (double)((t1 + 1023) / 1024));
+    p.mtiles = 4;
+    if (cost2 < cost4 && cost2 <= cost1) p.mtiles = 2;
+    else if (cost1 < cost4) p.mtiles = 1;
     if (m <= 32) p.mtiles = 1;
     if (mt_override == 1 || mt_override == 2 || mt_override == 4) p.mtiles = mt_override;
     const int64_t tiles = (int64_t)strips * ceil_div_i(m, 32 * p.mtiles);
