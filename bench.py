@@ -217,6 +217,50 @@ def sweep(dev, gen, out_path):
         print("fwht rows=%d dim=%d block=%d: %.2f us %.1f GB/s" % (rows_x, dim, block, sec * 1e6, per / sec / 1e9),
               file=sys.stderr, flush=True)
 
+    # MLP front act(gate(x)) * up(x): one launch with the epilogue against the product followed by
+    # torch's silu and multiply (random words are random interleaved gate/up weights just as well)
+    k, width = 4096, 14336
+    for m in (1, 8, 1024):
+        copies = copies_for(k * width) if m <= 64 else 2
+        weights = [make_weights(k, 2 * width, dev, gen) for _ in range(copies)]
+        x = torch.randn((m, k), device=dev, generator=gen).to(torch.float16)
+        ws = torch.zeros((2 * width // 64) * 16, dtype=torch.int32, device=dev)
+
+        def fused(i):
+            b, sc = weights[i % copies]
+            return ops.w4a16_linear(x, b, sc, ws, 2 * width, k, silu_mul=True)
+
+        def unfused(i):
+            b, sc = weights[i % copies]
+            y = ops.w4a16_linear(x, b, sc, ws, 2 * width, k).view(m, width // 64, 2, 64)
+            return torch.nn.functional.silu(y[:, :, 0]) * y[:, :, 1]
+
+        steps = 200 if m <= 64 else 20
+        sec_f, _ = time_graphs(fused, copies, steps, 20)
+        sec_u, _ = time_graphs(unfused, copies, steps, 20)
+        per = linear_bytes(m, k, 2 * width) - m * width * 2   # half the output bytes
+        rows.append(dict(op="gate_up_silu_mul", m=m, k=k, n=2 * width, us=sec_f * 1e6, us_unfused=sec_u * 1e6,
+                         gbs=per / sec_f / 1e9, tflops=linear_flops(m, k, 2 * width) / sec_f / 1e12))
+        print("gate_up + silu*mul M=%d: fused %.2f us (%.1f GB/s, %.1f TFLOP/s), product then torch ops %.2f us" % (
+            m, sec_f * 1e6, per / sec_f / 1e9, linear_flops(m, k, 2 * width) / sec_f / 1e12, sec_u * 1e6),
+            file=sys.stderr, flush=True)
+        del weights
+        torch.cuda.empty_cache()
+
+    # rotary embedding with gathered frequencies, Llama-3.1-8B heads (32 query, 8 key/value)
+    for rows_x, d in ((1, 128), (1024, 128), (1024, 108), (4096, 128)):
+        qs = [torch.randn((1, rows_x, 32, d), device=dev, generator=gen).to(torch.float16) for _ in range(4)]
+        ks = [torch.randn((1, rows_x, 8, d), device=dev, generator=gen).to(torch.float16) for _ in range(4)]
+        cos = torch.rand((1, rows_x, 128), device=dev, generator=gen).to(torch.float16)
+        sin = torch.rand((1, rows_x, 128), device=dev, generator=gen).to(torch.float16)
+        half = torch.arange(d // 2, device=dev)
+        idx = torch.cat((half, half + 64)).to(torch.uint8).repeat(8, 1)
+        sec, _ = time_graphs(lambda i: ops.rope_indices_(qs[i], ks[i], cos, sin, idx), 4, 200, 20)
+        per = rows_x * 40 * d * 2 * 2 + rows_x * 128 * 2 * 2
+        rows.append(dict(op="rope_indices", rows=rows_x, head_dim=d, us=sec * 1e6, gbs=per / sec / 1e9))
+        print("rope rows=%d head_dim=%d: %.2f us %.1f GB/s" % (rows_x, d, sec * 1e6, per / sec / 1e9),
+              file=sys.stderr, flush=True)
+
     os.makedirs(os.path.dirname(out_path), exist_ok=True)
     with open(out_path, "w") as f:
         json.dump(rows, f, indent=1)

@@ -95,6 +95,44 @@ int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, v
                      unsigned flags, void* stream);
 
 /*
+ * The whole forward of the reference's layer in one call, with the work around the product
+ * done inside the kernels instead of by separate tensor operations:
+ * W4A16B16O16Linear.forward (quantize/quant_linear_layers.py:92-114: pad the input to k,
+ * product, drop the padded output columns, add the bias), and, with UNIQL_EPI_SILU_MUL,
+ * the MLP's act_fn(gate_proj(x)) * up_proj(x) (modeling/llama/llama_qblocks.py:48-51).
+ * Arguments as uniql_w4a16_gemm, plus:
+ *   k_in      columns of A that exist (lda >= k_in, k_in % 8 == 0, k - 128 < k_in <= k); K rows
+ *             from k_in on count as zero activations (the module's pad_in)
+ *   bias      device, fp16 [n_out] in natural column order, or NULL; added to the fp16-rounded
+ *             product and rounded again, as the reference's `y + self.bias` does.  With
+ *             UNIQL_EPI_SILU_MUL: [2 n_out], the gate biases followed by the up biases
+ *   D, ldd    output rows of ldd elements (ldd >= n_out); 16-byte stores are used when
+ *             ldd % 8 == 0 and D is 16-byte aligned
+ *   n_out     output columns that exist (the module's out_features); the rest of n is dropped
+ *   epilogue  UNIQL_EPI_NONE: n_out <= n.
+ *             UNIQL_EPI_SILU_MUL: B and S hold the gate and the up projection interleaved in
+ *             blocks of 64 columns (block 2c = columns 64c.. of gate, block 2c+1 = the same
+ *             columns of up; packed words and permuted scales of a 64-column block are
+ *             contiguous, so this is a concatenation of slices of the two layers' tensors), n is
+ *             twice the padded width of one projection, n_out <= n/2, and
+ *             D[m, j] = fp16(fp16(silu(g)) * u) with g, u the fp16-rounded (and biased) gate and
+ *             up outputs of column j: the reference's sequence of roundings.
+ *   temp      uniql_w4a16_linear_temp_bytes(m, n, k, k_in, had_block) bytes
+ * With UNIQL_F_OUT_F32 D is float32 and no intermediate rounding is applied.
+ */
+enum { UNIQL_EPI_NONE = 0, UNIQL_EPI_SILU_MUL = 1 };
+
+size_t uniql_w4a16_linear_temp_bytes(int m, int n, int k, int k_in, int had_block);
+
+int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, const void* S, const void* bias,
+                       void* D, int64_t ldd, int n_out, int epilogue,
+                       const int32_t* workspace, int64_t workspace_len,
+                       void* accum, size_t accum_bytes, void* temp, size_t temp_bytes,
+                       int m, int n, int k, int groups,
+                       int had_block, float had_scale,
+                       unsigned flags, void* stream);
+
+/*
  * W[k, n] fp16 = fp16_rn((code - 8) * scale), natural (un-permuted) order.
  * The value csrc/linear/marlin_gemm_kernel.cuh:118-146 builds in registers and
  * quantize/quantize_helpers.py:118 calls w_ref.  Also writes the raw codes
@@ -149,6 +187,40 @@ int uniql_w4a16_pack(const uint8_t* codes, const void* scales, void* B, void* S,
 int uniql_w4_embedding_lookup(const int64_t* ids, int64_t ntokens,
                               const void* weight, const void* scales, void* out,
                               int64_t vocab, int dim, void* stream);
+
+/*
+ * Quantises an fp16 embedding table on the device: scales[v] = fp16(max|W[v, :]| / 8),
+ * code = clamp(round(W / scale + 8), 0, 15) with every operation rounded to fp16, eight codes
+ * per word in nibble order [0, 2, 4, 6, 1, 3, 5, 7].  Replaces the tensor arithmetic and the
+ * host packing loop of W4O16Embedding.from_fp16 (quantize/quant_embedding_layers.py:26-48)
+ * with the same results bit for bit.
+ *   W       device, fp16 [vocab, dim], row stride ldw elements (ldw % 8 == 0), 16-byte aligned
+ *   packed  device out, int32 [vocab, dim/8];  scales  device out, fp16 [vocab];  dim % 8 == 0
+ */
+int uniql_w4_embedding_quantize(const void* W, int64_t ldw, void* packed, void* scales,
+                                int64_t vocab, int dim, void* stream);
+
+/*
+ * Rotary position embedding with gathered frequencies, in place:
+ *   x[.., j] <- fp16(fp16(x[.., j] * cos[t, i(j)]) + fp16(rot(x)[.., j] * sin[t, i(j)]))
+ * with rot(x) = (-x[d/2:], x[:d/2]) and i(j) = indices[kv head of the head][j].  Replaces
+ * apply_rotary_pos_emb_indices_triton (modeling/rope_triton.py:10-177) with the arithmetic of
+ * the tensor version it stands in for (modeling/llama/llama_rope.py:38-96; the same function
+ * in modeling/qwen/qwen2_rope.py:37).
+ *   q        device, fp16 [rows, n_q_heads, head_dim], token-major (the projections' output
+ *            layout), rows = batch * seq_len, row stride q_row_stride elements; modified
+ *   k        device, fp16 [rows, n_kv_heads, head_dim], row stride k_row_stride; modified
+ *   cos,sin  device, fp16 [cos_batch, seq_len, cos_dim], row stride cos_row_stride;
+ *            cos_batch is 1 (all batches share the table) or the batch size
+ *   indices  device, [n_kv_heads, head_dim] integers of index_bytes (1: uint8 as the module
+ *            stores them, 4: int32, 8: int64), each < cos_dim; query head h uses row
+ *            h / (n_q_heads / n_kv_heads)
+ */
+int uniql_rope_indices(void* q, int64_t q_row_stride, void* k, int64_t k_row_stride,
+                       const void* cos, const void* sin, int64_t cos_row_stride,
+                       const void* indices, int index_bytes,
+                       int64_t rows, int seq_len, int cos_batch,
+                       int n_q_heads, int n_kv_heads, int head_dim, int cos_dim, void* stream);
 
 /*
  * y[r, :] = round((x[r, :] . H) * scale), H = Sylvester Hadamard matrix applied

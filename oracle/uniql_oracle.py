@@ -22,6 +22,12 @@ Pinning status (what proves each function right, besides reading):
     brute-force; the reference module cannot be imported without its compiled
     extension, so `embedding_quantize`'s code selection at exact rounding ties
     is "parity unpinned" beyond those cases
+  * module forward with its fp16 roundings, SiLU-gated MLP front (linear_forward_fp16,
+    silu_fp16, mlp_gate_up) ................. torch's own fp16 CPU operators over all
+    finite fp16 inputs / random tensors (the reference calls exactly those operators)
+  * rotary embedding with gathered frequencies (rope_indices) ... the textbook complex
+    rotation in float64 for identity indices, an independently permuted frequency table,
+    norm preservation, and torch's fp16 CPU arithmetic for the order of the roundings
   * power-of-two Hadamard .................... scipy.linalg.hadamard, involution,
     Parseval.  The 12N/20N/28N/40N variants need base matrices that live in an
     un-vendored third-party package (Dao-AILab fast-hadamard-transform, commit
@@ -266,6 +272,36 @@ def linear_forward(x: np.ndarray, packed: np.ndarray, scale_perm: np.ndarray, *,
     return y
 
 
+def linear_forward_fp16(x: np.ndarray, packed: np.ndarray, scale_perm: np.ndarray, *, in_features: int,
+                        out_features: int, bias: np.ndarray | None = None) -> np.ndarray:
+    """The module's fp16 result with its roundings: the kernel's fp32-accumulated product is
+    rounded to fp16 (marlin_gemm_kernel.cuh:560-606 writes halves), then `y + self.bias`
+    (quant_linear_layers.py:113-114) adds two fp16 tensors and rounds again.  The float64
+    product stands in for the fp32 accumulation (they differ by ~1e-6 relative)."""
+    y = linear_forward(x, packed, scale_perm, in_features=in_features, out_features=out_features,
+                       exact=True).astype(np.float16)
+    if bias is not None:
+        y = (y.astype(np.float32) + np.asarray(bias, dtype=np.float16).astype(np.float32)).astype(np.float16)
+    return y
+
+
+def silu_fp16(x: np.ndarray) -> np.ndarray:
+    """torch.nn.SiLU on an fp16 tensor (ACT2FN["silu"], llama_qblocks.py:36): the value is
+    computed in fp32 as x / (1 + exp(-x)) and rounded to fp16."""
+    x32 = np.asarray(x, dtype=np.float16).astype(np.float32)
+    with np.errstate(over="ignore"):
+        return (x32 / (np.float32(1.0) + np.exp(-x32))).astype(np.float16)
+
+
+def mlp_gate_up(gate16: np.ndarray, up16: np.ndarray) -> np.ndarray:
+    """act_fn(gate_proj(x)) * up_proj(x) on the two layers' fp16 outputs
+    (llama_qblocks.py:48-49): SiLU rounds to fp16, the product of two fp16 tensors rounds
+    again."""
+    a = silu_fp16(gate16).astype(np.float32)
+    with np.errstate(over="ignore"):
+        return (a * np.asarray(up16, dtype=np.float16).astype(np.float32)).astype(np.float16)
+
+
 # --------------------------------------------------------------------------
 # a10/a11: int4 embedding with one scale per vocabulary row
 # --------------------------------------------------------------------------
@@ -384,3 +420,37 @@ def linear_geometry(in_features: int, out_features: int, group_size: int = GROUP
                 workspace=(size_n // MIN_THREAD_N) * MAX_PARALLEL,
                 weight=(size_k // 16, size_n * 16 // 8),
                 scale=(size_k // group_size, size_n))
+
+
+# --------------------------------------------------------------------------
+# rotary embedding with per-head gathered frequencies (pruned attention heads)
+# --------------------------------------------------------------------------
+def rope_indices(q: np.ndarray, k: np.ndarray, cos: np.ndarray, sin: np.ndarray, indices: np.ndarray):
+    """apply_rotary_pos_emb_indices (modeling/llama/llama_rope.py:38-96) on fp16 arrays.
+
+    q [b, hq, s, d], k [b, hk, s, d]; cos, sin [b or 1, s, D] (D = the unpruned head width);
+    indices [hk, d] integer: which of the D table columns each kept column of a key/value head
+    uses; query head h uses row h // (hq / hk) (repeat_interleave, :80).
+    out = x * cos_g + rotate_half(x) * sin_g with every product and the sum rounded to fp16,
+    as torch does for fp16 tensors (:94-95; rotate_half :4-8 negates the upper half exactly).
+    """
+    q = np.asarray(q, dtype=np.float16)
+    k = np.asarray(k, dtype=np.float16)
+    b, hq, s, d = q.shape
+    hk = k.shape[1]
+    assert indices.shape == (hk, d) and hq % hk == 0
+    idx = np.asarray(indices, dtype=np.int64)
+    cos = np.broadcast_to(np.asarray(cos, dtype=np.float16), (b, s, cos.shape[-1]))
+    sin = np.broadcast_to(np.asarray(sin, dtype=np.float16), (b, s, sin.shape[-1]))
+
+    def rotate(x, head_rows):
+        # cos_g[b, h, s, j] = cos[b, s, idx[row(h), j]]
+        cg = np.transpose(cos[:, :, idx[head_rows]], (0, 2, 1, 3)).astype(np.float32)
+        sg = np.transpose(sin[:, :, idx[head_rows]], (0, 2, 1, 3)).astype(np.float32)
+        half = d // 2
+        rot = np.concatenate((-x[..., half:], x[..., :half]), axis=-1).astype(np.float32)
+        a = (x.astype(np.float32) * cg).astype(np.float16)
+        r = (rot * sg).astype(np.float16)
+        return (a.astype(np.float32) + r.astype(np.float32)).astype(np.float16)
+
+    return rotate(q, np.arange(hq) // (hq // hk)), rotate(k, np.arange(hk))

@@ -17,6 +17,7 @@ F_FORCE_SKINNY = 1 << 1
 F_FORCE_TILED = 1 << 2
 F_TRANSPOSE_OUT = 1 << 3
 DT_F16, DT_BF16, DT_F32 = 0, 1, 2
+EPI_NONE, EPI_SILU_MUL = 0, 1
 
 # every exported symbol with (restype, argtypes); tests check the list against the header
 SIGNATURES = {
@@ -27,12 +28,20 @@ SIGNATURES = {
     "uniql_w4a16_gemm": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
                                  c_void_p, c_int64, c_void_p, c_size_t, c_void_p, c_size_t,
                                  c_int, c_int, c_int, c_int, c_int, c_float, c_uint, c_void_p]),
+    "uniql_w4a16_linear_temp_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "uniql_w4a16_linear": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p,
+                                   c_void_p, c_int64, c_int, c_int,
+                                   c_void_p, c_int64, c_void_p, c_size_t, c_void_p, c_size_t,
+                                   c_int, c_int, c_int, c_int, c_int, c_float, c_uint, c_void_p]),
     "uniql_w4a16_dequant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "uniql_w4a16_quantize": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_void_p]),
     "uniql_w4a16_pack": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "uniql_w4_embedding_lookup": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
                                           c_int64, c_int, c_void_p]),
+    "uniql_w4_embedding_quantize": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
+    "uniql_rope_indices": (c_int, [c_void_p, c_int64, c_void_p, c_int64, c_void_p, c_void_p, c_int64,
+                                   c_void_p, c_int, c_int64, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
     "uniql_fwht": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_float, c_int, c_void_p]),
 }
 

@@ -3,17 +3,23 @@
 #include "common.hpp"
 
 namespace uniql {
-int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, void* accum, int m, int n,
-                  int k, int groups, bool had128, float had_scale, bool out_f32, unsigned tune,
-                  hipStream_t stream);
+int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const void* S, void* D,
+                  const Epilogue& epi, void* accum, int m, int n, int k, int groups, bool had128, float had_scale,
+                  unsigned tune, hipStream_t stream);
 size_t stream_accum_bytes(int m, int n, int k);
-int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, void* accum, size_t accum_bytes,
-                int m, int n, int k, int groups, bool out_f32, unsigned tune, hipStream_t stream);
+int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, const Epilogue& epi, void* accum,
+                size_t accum_bytes, int m, int n, int k, int groups, unsigned tune, hipStream_t stream);
+int pad_rows_launch(const void* A, int64_t lda, int k_in, void* dst, int k, int m, hipStream_t stream);
 size_t tile_accum_bytes(int m, int n, int k);
 int dequant_launch(const void* B, const void* S, void* W, uint8_t* codes, int n, int k, int groups,
                    hipStream_t stream);
 int embedding_launch(const int64_t* ids, int64_t ntokens, const void* weight, const void* scales, void* out,
                      int64_t vocab, int dim, hipStream_t stream);
+int embedding_quantize_launch(const void* W, int64_t ldw, void* packed, void* scales, int64_t vocab, int dim,
+                              hipStream_t stream);
+int rope_indices_launch(void* q, int64_t q_row_stride, void* k, int64_t k_row_stride, const void* cos, const void* sin,
+                        int64_t cos_row_stride, const void* indices, int index_bytes, int64_t rows, int seq_len,
+                        int cos_batch, int n_qh, int n_kh, int hd, hipStream_t stream);
 int fwht_launch(const void* x, void* y, int64_t rows, int dim, int block, float scale, int dtype,
                 hipStream_t stream);
 int quantize_launch(const void* W, int64_t ldw, const void* given_scales, void* B, void* S, int out_features,
@@ -62,31 +68,41 @@ size_t uniql_w4a16_gemm_accum_bytes(int m, int n, int k) {
     return round256(a > b ? a : b);
 }
 
-size_t uniql_w4a16_gemm_temp_bytes(int m, int n, int k, int had_block) {
+size_t uniql_w4a16_linear_temp_bytes(int m, int n, int k, int k_in, int had_block) {
     if (m <= 0 || n <= 0 || k <= 0) return 0;
-    // rotated activations: every block width except the 128 fused into the streaming kernel,
-    // and 128 too once the tiled kernel may take the call
-    if (had_block != 0) return round256((size_t)m * k * sizeof(half_t));
+    // a rotated (every block width except the 128 fused into the streaming kernel, and 128 too
+    // once the tiled kernel may take the call) or zero-padded copy of the activations
+    if (had_block != 0 || k_in != k) return round256((size_t)m * k * sizeof(half_t));
     return 0;
 }
 
-int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, void* D, const int32_t* workspace,
-                     int64_t workspace_len, void* accum, size_t accum_bytes, void* temp, size_t temp_bytes, int m,
-                     int n, int k, int groups, int had_block, float had_scale, unsigned flags, void* stream) {
+size_t uniql_w4a16_gemm_temp_bytes(int m, int n, int k, int had_block) {
+    return uniql_w4a16_linear_temp_bytes(m, n, k, k, had_block);
+}
+
+int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, const void* S, const void* bias,
+                       void* D, int64_t ldd, int n_out, int epilogue, const int32_t* workspace,
+                       int64_t workspace_len, void* accum, size_t accum_bytes, void* temp, size_t temp_bytes, int m,
+                       int n, int k, int groups, int had_block, float had_scale, unsigned flags, void* stream) {
     const int rc = check_linear_shape(m, n, k, groups);
     if (rc != UNIQL_OK) return rc;
     if (flags & UNIQL_F_TRANSPOSE_OUT) return UNIQL_E_UNSUPPORTED;
+    if (epilogue != UNIQL_EPI_NONE && epilogue != UNIQL_EPI_SILU_MUL) return UNIQL_E_UNSUPPORTED;
+    const bool gated = epilogue == UNIQL_EPI_SILU_MUL;
+    if (k_in <= 0 || k_in > k || k - k_in >= 128 || (k_in % 8) != 0) return UNIQL_E_SHAPE;
+    if (n_out <= 0 || n_out > (gated ? n / 2 : n) || ldd < n_out) return UNIQL_E_SHAPE;
     if (m == 0) return UNIQL_OK;
     if (!A || !B || !S || !D) return UNIQL_E_NULL;
-    if (lda < k || (lda % 8) != 0) return UNIQL_E_ALIGN;
-    if (!aligned16(A) || !aligned16(B) || !aligned16(S) || !aligned16(D)) return UNIQL_E_ALIGN;
+    if (lda < k_in || (lda % 8) != 0) return UNIQL_E_ALIGN;
+    const bool out_f32 = (flags & UNIQL_F_OUT_F32) != 0;
+    if (!aligned16(A) || !aligned16(B) || !aligned16(S)) return UNIQL_E_ALIGN;
+    if (reinterpret_cast<uintptr_t>(D) % (out_f32 ? 4 : 2) != 0) return UNIQL_E_ALIGN;
+    if (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)) return UNIQL_E_ALIGN;
     if (workspace && workspace_len < n / 128) return UNIQL_E_WORKSPACE;
     if (had_block != 0 && (!is_pow2(had_block) || had_block < 2 || had_block > 32768 || k % had_block != 0))
         return UNIQL_E_SHAPE;
     const size_t need_accum = uniql_w4a16_gemm_accum_bytes(m, n, k);
     if (need_accum > 0 && (!accum || accum_bytes < need_accum)) return UNIQL_E_WORKSPACE;
-    const size_t need_temp = uniql_w4a16_gemm_temp_bytes(m, n, k, had_block);
-    if (need_temp > 0 && (!temp || temp_bytes < need_temp)) return UNIQL_E_WORKSPACE;
     if ((accum && !aligned16(accum)) || (temp && !aligned16(temp))) return UNIQL_E_ALIGN;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
 
@@ -96,29 +112,56 @@ int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, v
 
     const void* Ain = A;
     int64_t ld = lda;
+    int k_valid = k_in;
     const bool had128 = (had_block == 128) && use_stream;
-    if (had_block != 0 && !had128) {
-        // rotate into the temporary buffer, then run the plain product on it
-        if (lda != k) {
+    const bool rotate_first = had_block != 0 && !had128;
+    const bool pad_first = k_in != k && (rotate_first || !use_stream);
+    if (rotate_first || pad_first) {
+        if (!temp || temp_bytes < round256((size_t)m * k * sizeof(half_t))) return UNIQL_E_WORKSPACE;
+    }
+    if (pad_first) {
+        const int e = pad_rows_launch(A, lda, k_in, temp, k, m, st);
+        if (e != UNIQL_OK) return e;
+        Ain = temp;
+        ld = k;
+        k_valid = k;
+    }
+    if (rotate_first) {
+        // rotate into the temporary buffer (in place when the padded copy is already there),
+        // then run the plain product on it
+        if (ld != k) {
             for (int r = 0; r < m; ++r) {
-                const int e = fwht_launch(reinterpret_cast<const half_t*>(A) + (size_t)r * lda,
+                const int e = fwht_launch(reinterpret_cast<const half_t*>(Ain) + (size_t)r * ld,
                                           reinterpret_cast<half_t*>(temp) + (size_t)r * k, 1, k, had_block, had_scale,
                                           UNIQL_DT_F16, st);
                 if (e != UNIQL_OK) return e;
             }
         } else {
-            const int e = fwht_launch(A, temp, m, k, had_block, had_scale, UNIQL_DT_F16, st);
+            const int e = fwht_launch(Ain, temp, m, k, had_block, had_scale, UNIQL_DT_F16, st);
             if (e != UNIQL_OK) return e;
         }
         Ain = temp;
         ld = k;
     }
+    Epilogue epi;
+    epi.bias = reinterpret_cast<const half_t*>(bias);
+    epi.ldd = ldd;
+    epi.n_store = n_out;
+    epi.gated = gated ? 1 : 0;
+    epi.out_f32 = out_f32 ? 1 : 0;
+    epi.vec_ok = (ldd % 8 == 0 && aligned16(D)) ? 1 : 0;
     const unsigned tune = flags >> 8;  // tuning fields, see the header
     if (use_stream)
-        return stream_launch(Ain, ld, B, S, D, accum, m, n, k, groups, had128, had_scale,
-                             (flags & UNIQL_F_OUT_F32) != 0, tune, st);
-    return tile_launch(Ain, ld, B, S, D, accum, accum_bytes, m, n, k, groups, (flags & UNIQL_F_OUT_F32) != 0, tune,
-                       st);
+        return stream_launch(Ain, ld, k_valid, B, S, D, epi, accum, m, n, k, groups, had128, had_scale, tune, st);
+    return tile_launch(Ain, ld, B, S, D, epi, accum, accum_bytes, m, n, k, groups, tune, st);
+}
+
+int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, void* D, const int32_t* workspace,
+                     int64_t workspace_len, void* accum, size_t accum_bytes, void* temp, size_t temp_bytes, int m,
+                     int n, int k, int groups, int had_block, float had_scale, unsigned flags, void* stream) {
+    if (D && !aligned16(D)) return UNIQL_E_ALIGN;
+    return uniql_w4a16_linear(A, lda, k, B, S, nullptr, D, n, n, UNIQL_EPI_NONE, workspace, workspace_len, accum,
+                              accum_bytes, temp, temp_bytes, m, n, k, groups, had_block, had_scale, flags, stream);
 }
 
 int uniql_w4a16_dequant(const void* B, const void* S, void* W, uint8_t* codes, int n, int k, int groups,
@@ -156,6 +199,36 @@ int uniql_w4_embedding_lookup(const int64_t* ids, int64_t ntokens, const void* w
     if (!ids || !weight || !scales || !out) return UNIQL_E_NULL;
     if (!aligned16(out) || (reinterpret_cast<uintptr_t>(weight) & 3u)) return UNIQL_E_ALIGN;
     return embedding_launch(ids, ntokens, weight, scales, out, vocab, dim, reinterpret_cast<hipStream_t>(stream));
+}
+
+int uniql_w4_embedding_quantize(const void* W, int64_t ldw, void* packed, void* scales, int64_t vocab, int dim,
+                                void* stream) {
+    if (vocab < 0 || dim <= 0 || dim % 8 != 0 || ldw < dim || ldw % 8 != 0) return UNIQL_E_SHAPE;
+    if (vocab == 0) return UNIQL_OK;
+    if (!W || !packed || !scales) return UNIQL_E_NULL;
+    if (!aligned16(W) || (reinterpret_cast<uintptr_t>(packed) & 3u)) return UNIQL_E_ALIGN;
+    return embedding_quantize_launch(W, ldw, packed, scales, vocab, dim, reinterpret_cast<hipStream_t>(stream));
+}
+
+int uniql_rope_indices(void* q, int64_t q_row_stride, void* k, int64_t k_row_stride, const void* cos,
+                       const void* sin, int64_t cos_row_stride, const void* indices, int index_bytes, int64_t rows,
+                       int seq_len, int cos_batch, int n_q_heads, int n_kv_heads, int head_dim, int cos_dim,
+                       void* stream) {
+    if (rows < 0 || seq_len <= 0 || n_q_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0 || cos_dim <= 0)
+        return UNIQL_E_SHAPE;
+    if (head_dim % 2 != 0 || n_q_heads % n_kv_heads != 0) return UNIQL_E_SHAPE;
+    if (index_bytes != 1 && index_bytes != 4 && index_bytes != 8) return UNIQL_E_UNSUPPORTED;
+    if (index_bytes == 1 && cos_dim > 256) return UNIQL_E_SHAPE;
+    if (cos_batch != 1 && (cos_batch <= 0 || rows != (int64_t)cos_batch * seq_len)) return UNIQL_E_SHAPE;
+    if (cos_batch == 1 && rows % seq_len != 0) return UNIQL_E_SHAPE;
+    if (q_row_stride < (int64_t)n_q_heads * head_dim || k_row_stride < (int64_t)n_kv_heads * head_dim ||
+        cos_row_stride < cos_dim)
+        return UNIQL_E_SHAPE;
+    if (rows == 0) return UNIQL_OK;
+    if (!q || !k || !cos || !sin || !indices) return UNIQL_E_NULL;
+    return rope_indices_launch(q, q_row_stride, k, k_row_stride, cos, sin, cos_row_stride, indices, index_bytes,
+                               rows, seq_len, cos_batch, n_q_heads, n_kv_heads, head_dim,
+                               reinterpret_cast<hipStream_t>(stream));
 }
 
 int uniql_fwht(const void* x, void* y, int64_t rows, int dim, int block, float scale, int dtype, void* stream) {

@@ -79,6 +79,106 @@ __device__ __forceinline__ int single_scale_pos(int n) {
     return blk + 8 * ((c & 7) >> 1) + 2 * (c >> 3) + (c & 1);
 }
 
+// ---- what happens to a finished output element --------------------------------------
+// The reference's layer rounds the product to fp16, drops the padding columns, then adds the
+// fp16 bias (second rounding); its MLP applies SiLU to the fp16 gate output (third rounding)
+// and multiplies by the fp16 up output (fourth).  The same roundings are made here, in
+// registers, so that the fused result equals the unfused sequence.
+struct Epilogue {
+    const half_t* bias;  // natural order [n_store] (gated: gate biases, then up biases), or nullptr
+    int64_t ldd;         // elements between output rows
+    int n_store;         // output columns that exist; columns from here on are dropped
+    int gated;           // 1: columns c and c + 64 of a 128-column strip are the gate and up values
+                         //    of output column 64 strip + c; the output is silu(gate) * up
+    int out_f32;         // D is float32 and receives the values before any rounding
+    int vec_ok;          // ldd and D allow 16-byte stores of eight fp16 outputs
+};
+
+__device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
+
+// value of output column n (< n_store) from its fp32 product, and of a gated pair
+__device__ __forceinline__ half_t finish_half(const Epilogue& e, int n, float v) {
+    half_t y = (half_t)v;
+    if (e.bias) y = (half_t)((float)y + (float)e.bias[n]);
+    return y;
+}
+__device__ __forceinline__ half_t finish_half_gated(const Epilogue& e, int n, float g, float u) {
+    const half_t g16 = finish_half(e, n, g);
+    half_t u16 = (half_t)u;
+    if (e.bias) u16 = (half_t)((float)u16 + (float)e.bias[e.n_store + n]);
+    const half_t a16 = (half_t)silu_f32((float)g16);
+    return (half_t)((float)a16 * (float)u16);
+}
+
+__device__ __forceinline__ void finish_store(const Epilogue& e, void* D, int m, int n, float v) {
+    if (n >= e.n_store) return;
+    const size_t o = (size_t)m * e.ldd + n;
+    if (e.out_f32)
+        reinterpret_cast<float*>(D)[o] = e.bias ? v + (float)e.bias[n] : v;
+    else
+        reinterpret_cast<half_t*>(D)[o] = finish_half(e, n, v);
+}
+
+__device__ __forceinline__ void finish_store_gated(const Epilogue& e, void* D, int m, int n, float g, float u) {
+    if (n >= e.n_store) return;
+    const size_t o = (size_t)m * e.ldd + n;
+    if (e.out_f32) {
+        if (e.bias) {
+            g += (float)e.bias[n];
+            u += (float)e.bias[e.n_store + n];
+        }
+        reinterpret_cast<float*>(D)[o] = silu_f32(g) * u;
+    } else {
+        reinterpret_cast<half_t*>(D)[o] = finish_half_gated(e, n, g, u);
+    }
+}
+
+// ---- exchange of partial sums between workgroups that split K ------------------------
+// One 64-bit word per output element in a zero-initialised buffer: bits 8..63 the running sum
+// in units of 2^-24, bits 0..7 the number of contributions.  Integer adds commute, so the total
+// does not depend on arrival order.
+constexpr float kAccumScale = 16777216.0f;  // 2^24 fixed-point units per 1.0
+constexpr float kAccumClamp = 4194304.0f;   // 2^22: far beyond the fp16 range of the outputs
+
+__device__ __forceinline__ unsigned long long accum_word(float v, unsigned count) {
+    const float c = fminf(fmaxf(v, -kAccumClamp), kAccumClamp);
+    return ((unsigned long long)__float2ll_rn(c * kAccumScale) << 8) + count;
+}
+__device__ __forceinline__ float accum_value(unsigned long long word) {
+    return (float)((long long)word >> 8) * (1.0f / kAccumScale);
+}
+// Adds one contribution.  True for the last of `splits` arrivals, which gets the total and
+// must put the word back to zero (accum_reset) after using it.
+__device__ __forceinline__ bool accum_add(unsigned long long* p, float v, int splits, float& total) {
+    const unsigned long long word = accum_word(v, 1u);
+    const unsigned long long old = __hip_atomic_fetch_add(p, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((int)(old & 0xffull) != splits - 1) return false;
+    total = accum_value(old + word);
+    return true;
+}
+__device__ __forceinline__ void accum_reset(unsigned long long* p) {
+    __hip_atomic_store(p, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// Gated pair: the up value is added first (its word carries no count); the gate word's add is
+// issued only after the up add has returned, i.e. has been performed.  Whoever completes the
+// gate word's count therefore finds every up contribution in place and takes it with an
+// exchange, which also leaves that word zero.
+__device__ __forceinline__ bool accum_add_pair(unsigned long long* pg, unsigned long long* pu, float g, float u,
+                                               int splits, float& total_g, float& total_u) {
+    const unsigned long long old_u =
+        __hip_atomic_fetch_add(pu, accum_word(u, 0u), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    unsigned long long word = accum_word(g, 1u);
+    uint32_t lo = (uint32_t)word;
+    const uint32_t returned = (uint32_t)old_u;
+    asm volatile("" : "+v"(lo) : "v"(returned));  // the gate word now depends on the up add's return value
+    word = (word & 0xffffffff00000000ull) | lo;
+    const unsigned long long old = __hip_atomic_fetch_add(pg, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if ((int)(old & 0xffull) != splits - 1) return false;
+    total_g = accum_value(old + word);
+    total_u = accum_value(__hip_atomic_exchange(pu, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    return true;
+}
+
 // Butterflies of a 128-point Walsh-Hadamard transform on a row spread over 16
 // consecutive lanes, 8 consecutive elements per lane (element e = 8*seg + i).
 // In-lane stages handle index bits 0..2, lane exchanges handle bits 3..6.

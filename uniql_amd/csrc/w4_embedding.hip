@@ -49,6 +49,66 @@ __global__ __launch_bounds__(256) void w4_embedding_kernel(const int64_t* __rest
     }
 }
 
+// Producer side: one workgroup quantises one table row.  scale = fp16(max|w| / 8),
+// code = clamp(round(fp16(fp16(w / scale) + 8)), 0, 15): every operation rounded to fp16 as
+// the tensor expression of the reference does on an fp16 table
+// (quantize/quant_embedding_layers.py:35-37).  An all-zero row divides 0 by 0: the NaN
+// becomes code 0 (the reference's NaN -> int32 -> uint32 conversion leaves the low nibble 0).
+// Element 2 p + odd of every eight goes to nibble 4 odd + p of the word (:33,39-43).
+__global__ __launch_bounds__(256) void w4_embedding_quantize_kernel(const half_t* __restrict__ W, int64_t ldw,
+                                                                   uint32_t* __restrict__ packed,
+                                                                   half_t* __restrict__ scales, int words) {
+    __shared__ float wave_max[4];
+    const int64_t row = blockIdx.x;
+    const half_t* src = W + row * ldw;
+    float amax = 0.f;
+    for (int w = threadIdx.x; w < words; w += 256) {
+        const h8 v = *reinterpret_cast<const h8*>(src + 8 * w);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const float f = fabsf((float)v[i]);
+            amax = (f > amax || f != f) ? f : amax;  // a NaN in the row makes the scale NaN, as amax() does
+        }
+    }
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const float o = __shfl_xor(amax, d, kWave);
+        amax = (o > amax || o != o) ? o : amax;
+    }
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = amax;
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const float o = wave_max[i];
+        amax = (o > amax || o != o) ? o : amax;
+    }
+    const half_t scale = (half_t)(amax / 8.0f);
+    if (threadIdx.x == 0) scales[row] = scale;
+    for (int w = threadIdx.x; w < words; w += 256) {
+        const h8 v = *reinterpret_cast<const h8*>(src + 8 * w);
+        uint32_t word = 0u;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const half_t q = (half_t)((float)v[i] / (float)scale);
+            const half_t shifted = (half_t)((float)q + 8.0f);
+            const float r = __builtin_rintf((float)shifted);
+            const uint32_t code = (uint32_t)fminf(fmaxf(r, 0.0f), 15.0f);  // fmaxf(NaN, 0) = 0
+            word |= code << (4 * (4 * (i & 1) + (i >> 1)));
+        }
+        packed[row * words + w] = word;
+    }
+}
+
+int embedding_quantize_launch(const void* W, int64_t ldw, void* packed, void* scales, int64_t vocab, int dim,
+                              hipStream_t stream) {
+    if (vocab == 0) return UNIQL_OK;
+    if (vocab > 0x7fffffffLL) return UNIQL_E_SHAPE;
+    hipLaunchKernelGGL(w4_embedding_quantize_kernel, dim3((unsigned)vocab), dim3(256), 0, stream,
+                       reinterpret_cast<const half_t*>(W), ldw, reinterpret_cast<uint32_t*>(packed),
+                       reinterpret_cast<half_t*>(scales), dim / 8);
+    return hipGetLastError() == hipSuccess ? UNIQL_OK : UNIQL_E_LAUNCH;
+}
+
 int embedding_launch(const int64_t* ids, int64_t ntokens, const void* weight, const void* scales, void* out,
                      int64_t vocab, int dim, hipStream_t stream) {
     if (ntokens == 0) return UNIQL_OK;

@@ -43,15 +43,13 @@
 
 namespace uniql {
 
-constexpr float kAccumScale = 16777216.0f;  // 2^24 fixed-point units per 1.0
-constexpr float kAccumClamp = 4194304.0f;   // 2^22
 constexpr int kXsStride = 68;  // dwords per staged activation row: 64 + 4, keeps the 64 lanes on distinct banks
 
 struct StreamArgs {
     const u32x4* B;       // packed weights, [K/16][N/2] 16-byte pieces
     const half_t* S;      // permuted scales [groups][N]
     const half_t* X;      // activations [M][ldx]
-    void* D;              // fp16 or fp32 [M][N]
+    void* D;              // fp16 or fp32 [M][epi.ldd]
     unsigned long long* accum;  // [M][N] fixed-point sum | count words, zero on entry and on exit (splits > 1)
     int64_t ldx;
     int M, N, K;
@@ -60,16 +58,10 @@ struct StreamArgs {
     int upw;              // groups per wave
     int splits;           // workgroups along K per strip
     int xrows;            // activation rows staged per wave: multiple of 4, >= min(M, 16 MT)
-    int out_f32;
+    int k_valid;          // columns of X that exist (multiple of 8); the rest of K counts as zeros
     float had_scale;
+    Epilogue epi;
 };
-
-__device__ __forceinline__ void store_out(const StreamArgs& a, int m, int n, float v) {
-    if (a.out_f32)
-        reinterpret_cast<float*>(a.D)[(size_t)m * a.N + n] = v;
-    else
-        reinterpret_cast<half_t*>(a.D)[(size_t)m * a.N + n] = (half_t)v;
-}
 
 // MT: 16-row tiles of M per workgroup.  RC: row class, an upper bound of M for MT = 1
 // (1, 2, 4, 8, 16): it fixes NV, how many of the four output rows of a lane's accumulator
@@ -77,8 +69,11 @@ __device__ __forceinline__ void store_out(const StreamArgs& a, int m, int n, flo
 // wavefronts per workgroup (4 or 8); with 8 a workgroup can cover all of K for shapes with
 // many strips, which removes the exchange of partial sums between workgroups.  A wave keeps one
 // group's weights in registers at a time: a second register set for the next group costs more
-// in occupancy than it hides in latency, the other waves of the SIMD do that.
-template <int MT, int RC, bool HAD, int WAVES>
+// in occupancy than it hides in latency, the other waves of the SIMD do that.  EXT: the call
+// uses something beyond the plain product (input shorter than K, output cut or strided, bias,
+// gated pairs); the plain instantiation leaves all of that code out, which at a few
+// microseconds per launch is measurable (instruction fetch).
+template <int MT, int RC, bool HAD, int WAVES, bool EXT>
 __global__ __launch_bounds__(64 * WAVES, (MT == 1 ? 3 : (MT == 2 ? 2 : 1)))
 void w4a16_stream_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
@@ -147,7 +142,7 @@ void w4a16_stream_kernel(const StreamArgs a) {
             for (int i = 0; i < XQ; ++i) {
                 const int m = mt * 16 + i * 4 + kq;
                 xv[mt][i] = u32x4{0u, 0u, 0u, 0u};
-                if (m < a.M)
+                if (m < a.M && (!EXT || 128 * g + 8 * slot < a.k_valid))
                     xv[mt][i] = *reinterpret_cast<const u32x4*>(a.X + (size_t)m * a.ldx + 128 * g + 8 * slot);
             }
         }
@@ -285,12 +280,14 @@ void w4a16_stream_kernel(const StreamArgs a) {
     const int ncol_lane = 64 * (slot >> 3) + c8;
     const int col_out = tid & 127;
     const int n_out = 128 * strip + col_out;
+    const bool gated = EXT && a.epi.gated != 0;  // uniform
+    const int col_pair = col_out ^ 64;    // the other half of a (gate, up) pair
     bool first_round = true;
     for (int mt = 0; mt < MT; ++mt) {
         if (mt * 16 >= a.M) break;
-        float tot[NI];
+        float tot[NI], oth[NI];
 #pragma unroll
-        for (int i = 0; i < NI; ++i) tot[i] = 0.f;
+        for (int i = 0; i < NI; ++i) tot[i] = oth[i] = 0.f;
         for (int round = 0; round < WAVES / wpr; ++round) {
             if (!first_round) __syncthreads();
             first_round = false;
@@ -311,29 +308,40 @@ void w4a16_stream_kernel(const StreamArgs a) {
             for (int i = 0; i < NI; ++i) {
                 const int ml = (tid >> 7) + RPT * i;
                 if (mt * 16 + ml < a.M) {
-                    for (int ww = 0; ww < wpr; ++ww) tot[i] += red[(ww * rr_rows + ml) * 128 + col_out];
+                    for (int ww = 0; ww < wpr; ++ww) {
+                        tot[i] += red[(ww * rr_rows + ml) * 128 + col_out];
+                        if (gated) oth[i] += red[(ww * rr_rows + ml) * 128 + col_pair];
+                    }
                 }
             }
         }
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             const int m = mt * 16 + (tid >> 7) + RPT * i;
-            if (m < a.M) {
+            if (m >= a.M) continue;
+            unsigned long long* word = a.accum + (size_t)m * a.N + n_out;
+            if (!gated) {
+                float total = tot[i];
+                const bool mine = a.splits == 1 || accum_add(word, tot[i], a.splits, total);
+                if (mine) {
+                    if constexpr (EXT) {
+                        finish_store(a.epi, a.D, m, n_out, total);
+                    } else if (a.epi.out_f32) {
+                        reinterpret_cast<float*>(a.D)[(size_t)m * a.N + n_out] = total;
+                    } else {
+                        reinterpret_cast<half_t*>(a.D)[(size_t)m * a.N + n_out] = (half_t)total;
+                    }
+                    if (a.splits != 1) accum_reset(word);
+                }
+            } else if (col_out < 64) {
+                const int n_pair = 64 * strip + col_out;
                 if (a.splits == 1) {
-                    store_out(a, m, n_out, tot[i]);
+                    finish_store_gated(a.epi, a.D, m, n_pair, tot[i], oth[i]);
                 } else {
-                    // fixed point: |v| is clamped to 2^22 (an fp16 result overflows long before),
-                    // so up to 255 contributions fit the 56-bit field
-                    const float v = fminf(fmaxf(tot[i], -kAccumClamp), kAccumClamp);
-                    const long long fixed = __float2ll_rn(v * kAccumScale);
-                    const unsigned long long word = ((unsigned long long)fixed << 8) + 1ull;
-                    unsigned long long* slot_ptr = a.accum + (size_t)m * a.N + n_out;
-                    const unsigned long long old =
-                        __hip_atomic_fetch_add(slot_ptr, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    if ((int)(old & 0xffull) == a.splits - 1) {
-                        const long long total = (long long)(old + word) >> 8;
-                        store_out(a, m, n_out, (float)total * (1.0f / kAccumScale));
-                        __hip_atomic_store(slot_ptr, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    float total_g, total_u;
+                    if (accum_add_pair(word, word + 64, tot[i], oth[i], a.splits, total_g, total_u)) {
+                        finish_store_gated(a.epi, a.D, m, n_pair, total_g, total_u);
+                        accum_reset(word);
                     }
                 }
             }
@@ -398,12 +406,12 @@ size_t stream_accum_bytes(int m, int n, int k) {
     return (size_t)mrows * n * sizeof(unsigned long long);
 }
 
-template <int MT, int RC, bool HAD, int WAVES>
+template <int MT, int RC, bool HAD, int WAVES, bool EXT>
 static hipError_t launch_one(const StreamArgs& a, hipStream_t stream) {
     const size_t stage = (size_t)WAVES * a.xrows * kXsStride * 4;
     const size_t red = a.xrows <= 4 ? (size_t)WAVES * 4 * 128 * 4 : (size_t)4 * 16 * 128 * 4;
     const size_t shmem = stage + red;
-    auto kern = &w4a16_stream_kernel<MT, RC, HAD, WAVES>;
+    auto kern = &w4a16_stream_kernel<MT, RC, HAD, WAVES, EXT>;
     if (shmem > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -414,31 +422,37 @@ static hipError_t launch_one(const StreamArgs& a, hipStream_t stream) {
     return hipGetLastError();
 }
 
+// The plain instantiation exists for the decode shapes (one 16-row tile); larger tiles are only
+// reached by forcing this kernel and always take the full one.
 template <int MT, int RC, bool HAD>
-static hipError_t launch_waves(const StreamArgs& a, int waves, hipStream_t stream) {
+static hipError_t launch_waves(const StreamArgs& a, int waves, bool ext, hipStream_t stream) {
     if constexpr (MT == 1) {
-        if (waves == 8) return launch_one<MT, RC, HAD, 8>(a, stream);
+        if (waves == 8)
+            return ext ? launch_one<MT, RC, HAD, 8, true>(a, stream) : launch_one<MT, RC, HAD, 8, false>(a, stream);
+        return ext ? launch_one<MT, RC, HAD, 4, true>(a, stream) : launch_one<MT, RC, HAD, 4, false>(a, stream);
     }
-    return launch_one<MT, RC, HAD, 4>(a, stream);
+    return launch_one<MT, RC, HAD, 4, true>(a, stream);
 }
 
 template <bool HAD>
 static hipError_t launch_rows(const StreamArgs& a, int mt, int waves, hipStream_t stream) {
-    if (mt == 4) return launch_waves<4, 16, HAD>(a, waves, stream);
-    if (mt == 2) return launch_waves<2, 16, HAD>(a, waves, stream);
-    if (a.M == 1) return launch_waves<1, 1, HAD>(a, waves, stream);
-    if (a.M == 2) return launch_waves<1, 2, HAD>(a, waves, stream);
-    if (a.M <= 4) return launch_waves<1, 4, HAD>(a, waves, stream);
-    if (a.M <= 8) return launch_waves<1, 8, HAD>(a, waves, stream);
-    return launch_waves<1, 16, HAD>(a, waves, stream);
+    const Epilogue& e = a.epi;
+    const bool ext = e.gated || e.bias || e.n_store != a.N || e.ldd != a.N || a.k_valid != a.K;
+    if (mt == 4) return launch_waves<4, 16, HAD>(a, waves, ext, stream);
+    if (mt == 2) return launch_waves<2, 16, HAD>(a, waves, ext, stream);
+    if (a.M == 1) return launch_waves<1, 1, HAD>(a, waves, ext, stream);
+    if (a.M == 2) return launch_waves<1, 2, HAD>(a, waves, ext, stream);
+    if (a.M <= 4) return launch_waves<1, 4, HAD>(a, waves, ext, stream);
+    if (a.M <= 8) return launch_waves<1, 8, HAD>(a, waves, ext, stream);
+    return launch_waves<1, 16, HAD>(a, waves, ext, stream);
 }
 
 // Rows are processed in slabs of at most 64; every slab re-streams the weights.
 // tune: bits 0..7 groups per wave, bits 8..12 waves per workgroup (4 or 8); zero fields mean
 // "choose".
-int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, void* accum, int m, int n,
-                  int k, int groups, bool had128, float had_scale, bool out_f32, unsigned tune,
-                  hipStream_t stream) {
+int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const void* S, void* D,
+                  const Epilogue& epi, void* accum, int m, int n, int k, int groups, bool had128, float had_scale,
+                  unsigned tune, hipStream_t stream) {
     StreamArgs a;
     a.B = reinterpret_cast<const u32x4*>(B);
     a.S = reinterpret_cast<const half_t*>(S);
@@ -448,11 +462,12 @@ int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void
     a.K = k;
     a.G = k / 128;
     a.per_column = (groups == 1) ? 1 : 0;
-    a.out_f32 = out_f32 ? 1 : 0;
+    a.k_valid = k_valid;
+    a.epi = epi;
     a.had_scale = had_scale;
     int waves_override = (int)((tune >> 8) & 0x1fu);
     if (waves_override != 4 && waves_override != 8) waves_override = 0;
-    const size_t out_elt = out_f32 ? 4 : 2;
+    const size_t out_elt = epi.out_f32 ? 4 : 2;
     for (int m0 = 0; m0 < m; m0 += 64) {
         const int mm = (m - m0) < 64 ? (m - m0) : 64;
         const int mt = mm <= 16 ? 1 : (mm <= 32 ? 2 : 4);
@@ -462,7 +477,7 @@ int stream_launch(const void* A, int64_t lda, const void* B, const void* S, void
         a.M = mm;
         a.xrows = mt == 1 ? ((mm + 3) / 4) * 4 : mt * 16;
         a.X = reinterpret_cast<const half_t*>(A) + (size_t)m0 * lda;
-        a.D = reinterpret_cast<char*>(D) + (size_t)m0 * n * out_elt;
+        a.D = reinterpret_cast<char*>(D) + (size_t)m0 * epi.ldd * out_elt;
         const hipError_t e = had128 ? launch_rows<true>(a, mt, plan.waves, stream)
                                     : launch_rows<false>(a, mt, plan.waves, stream);
         if (e != hipSuccess) return UNIQL_E_LAUNCH;

@@ -39,8 +39,6 @@ namespace uniql {
 
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-constexpr float kTileAccumScale = 16777216.0f;  // 2^24
-constexpr float kTileAccumClamp = 4194304.0f;   // 2^22
 constexpr int kRing = 3;
 
 struct TileArgs {
@@ -56,7 +54,7 @@ struct TileArgs {
     int gps;          // K groups per split
     int splits;
     int mblocks;      // ceil(M / (32 MT))
-    int out_f32;
+    Epilogue epi;
 };
 
 typedef const __attribute__((address_space(1))) void* gptr_t;
@@ -64,6 +62,54 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 
 // s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding)
 #define UNIQL_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
+
+// Eight consecutive outputs of row m starting at column n0 (a multiple of 8): one 16-byte
+// store where the output's layout allows it, element stores otherwise.
+__device__ __forceinline__ void store_eight(const Epilogue& e, void* D, int m, int n0, f4 lo, f4 hi) {
+    if (e.vec_ok && n0 + 8 <= e.n_store) {
+        const size_t o = (size_t)m * e.ldd + n0;
+        if (e.out_f32 && !e.bias) {
+            float* d = reinterpret_cast<float*>(D) + o;
+            *reinterpret_cast<f4*>(d) = lo;
+            *reinterpret_cast<f4*>(d + 4) = hi;
+            return;
+        }
+        if (!e.out_f32) {
+            half_t r[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                r[i] = finish_half(e, n0 + i, lo[i]);
+                r[4 + i] = finish_half(e, n0 + 4 + i, hi[i]);
+            }
+            *reinterpret_cast<h8*>(reinterpret_cast<half_t*>(D) + o) = h8{r[0], r[1], r[2], r[3], r[4], r[5], r[6], r[7]};
+            return;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        finish_store(e, D, m, n0 + i, lo[i]);
+        finish_store(e, D, m, n0 + 4 + i, hi[i]);
+    }
+}
+__device__ __forceinline__ void store_eight_gated(const Epilogue& e, void* D, int m, int n0, f4 glo, f4 ghi, f4 ulo,
+                                                  f4 uhi) {
+    if (e.vec_ok && !e.out_f32 && n0 + 8 <= e.n_store) {
+        half_t r[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            r[i] = finish_half_gated(e, n0 + i, glo[i], ulo[i]);
+            r[4 + i] = finish_half_gated(e, n0 + 4 + i, ghi[i], uhi[i]);
+        }
+        *reinterpret_cast<h8*>(reinterpret_cast<half_t*>(D) + (size_t)m * e.ldd + n0) =
+            h8{r[0], r[1], r[2], r[3], r[4], r[5], r[6], r[7]};
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        finish_store_gated(e, D, m, n0 + i, glo[i], ulo[i]);
+        finish_store_gated(e, D, m, n0 + 4 + i, ghi[i], uhi[i]);
+    }
+}
 
 template <int MT>
 struct TileLds {
@@ -77,7 +123,9 @@ struct TileLds {
     static constexpr size_t kBytes = kRingBytes > kRedBytes ? kRingBytes : kRedBytes;
 };
 
-template <int MT>
+// EXT: the call uses something beyond the plain product (output cut or strided, bias, gated
+// pairs); the plain instantiation leaves that code out of the epilogue.
+template <int MT, bool EXT>
 __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     using L = TileLds<MT>;
@@ -355,6 +403,7 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     constexpr int kRedStride = 132;
     float* red = reinterpret_cast<float*>(lds);  // [4 waves][32 rows][132]
     const bool split_k = a.splits > 1;
+    const bool gated = EXT && a.epi.gated != 0;  // uniform
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         if (m0 + mt * 32 < a.M) {  // uniform
@@ -370,10 +419,13 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
             }
             __syncthreads();
             if (!split_k) {
-#pragma unroll
-                for (int u2 = 0; u2 < 2; ++u2) {
+                // gated: the 32 x 64 output block is 256 units, one per thread (columns c0 and
+                // c0 + 64 of the strip); else 512 units, two per thread
+                const int units = gated ? 1 : 2;
+                for (int u2 = 0; u2 < units; ++u2) {
                     const int unit = tid + 256 * u2;
-                    const int row = unit >> 4, c0 = (unit & 15) * 8;
+                    const int row = gated ? unit >> 3 : unit >> 4;
+                    const int c0 = gated ? (unit & 7) * 8 : (unit & 15) * 8;
                     const int m = m0 + mt * 32 + row;
                     const float* src = red + row * kRedStride + c0;
                     f4 lo = *reinterpret_cast<const f4*>(src), hi = *reinterpret_cast<const f4*>(src + 4);
@@ -382,18 +434,32 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
                         lo += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride);
                         hi += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride + 4);
                     }
-                    if (m < a.M) {
-                        const size_t o = (size_t)m * a.N + 128 * strip + c0;
-                        if (a.out_f32) {
-                            float* d = reinterpret_cast<float*>(a.D) + o;
-                            *reinterpret_cast<f4*>(d) = lo;
-                            *reinterpret_cast<f4*>(d + 4) = hi;
-                        } else {
-                            const h2 r0 = h2{(half_t)lo[0], (half_t)lo[1]}, r1 = h2{(half_t)lo[2], (half_t)lo[3]};
-                            const h2 r2 = h2{(half_t)hi[0], (half_t)hi[1]}, r3 = h2{(half_t)hi[2], (half_t)hi[3]};
-                            *reinterpret_cast<u32x4*>(reinterpret_cast<half_t*>(a.D) + o) =
-                                u32x4{h2_to_bits(r0), h2_to_bits(r1), h2_to_bits(r2), h2_to_bits(r3)};
+                    if (!gated) {
+                        if (m < a.M) {
+                            if constexpr (EXT) {
+                                store_eight(a.epi, a.D, m, 128 * strip + c0, lo, hi);
+                            } else {
+                                const size_t o = (size_t)m * a.N + 128 * strip + c0;
+                                if (a.epi.out_f32) {
+                                    float* d = reinterpret_cast<float*>(a.D) + o;
+                                    *reinterpret_cast<f4*>(d) = lo;
+                                    *reinterpret_cast<f4*>(d + 4) = hi;
+                                } else {
+                                    const h2 r0 = h2{(half_t)lo[0], (half_t)lo[1]}, r1 = h2{(half_t)lo[2], (half_t)lo[3]};
+                                    const h2 r2 = h2{(half_t)hi[0], (half_t)hi[1]}, r3 = h2{(half_t)hi[2], (half_t)hi[3]};
+                                    *reinterpret_cast<u32x4*>(reinterpret_cast<half_t*>(a.D) + o) =
+                                        u32x4{h2_to_bits(r0), h2_to_bits(r1), h2_to_bits(r2), h2_to_bits(r3)};
+                                }
+                            }
                         }
+                    } else {
+                        f4 ulo = *reinterpret_cast<const f4*>(src + 64), uhi = *reinterpret_cast<const f4*>(src + 68);
+#pragma unroll
+                        for (int ww = 1; ww < 4; ++ww) {
+                            ulo += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride + 64);
+                            uhi += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride + 68);
+                        }
+                        if (m < a.M) store_eight_gated(a.epi, a.D, m, 64 * strip + c0, lo, hi, ulo, uhi);
                     }
                 }
             } else {
@@ -403,23 +469,31 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
                 for (int i = 0; i < 16; ++i) {
                     const int row = (tid >> 7) + 2 * i;
                     const int m = m0 + mt * 32 + row;
-                    if (m < a.M) {
-                        const float* src = red + row * kRedStride + col_out;
-                        const float sum = (src[0] + src[32 * kRedStride]) + (src[64 * kRedStride] + src[96 * kRedStride]);
-                        const size_t o = (size_t)m * a.N + 128 * strip + col_out;
-                        const float v = fminf(fmaxf(sum, -kTileAccumClamp), kTileAccumClamp);
-                        const long long fixed = __float2ll_rn(v * kTileAccumScale);
-                        const unsigned long long word = ((unsigned long long)fixed << 8) + 1ull;
-                        unsigned long long* slot_ptr = a.accum + o;
-                        const unsigned long long old =
-                            __hip_atomic_fetch_add(slot_ptr, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                        if ((int)(old & 0xffull) == a.splits - 1) {
-                            const float outv = (float)((long long)(old + word) >> 8) * (1.0f / kTileAccumScale);
-                            if (a.out_f32)
-                                reinterpret_cast<float*>(a.D)[o] = outv;
-                            else
-                                reinterpret_cast<half_t*>(a.D)[o] = (half_t)outv;
-                            __hip_atomic_store(slot_ptr, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    if (m >= a.M) continue;
+                    const float* src = red + row * kRedStride + col_out;
+                    const float sum = (src[0] + src[32 * kRedStride]) + (src[64 * kRedStride] + src[96 * kRedStride]);
+                    const int n_out = 128 * strip + col_out;
+                    unsigned long long* word = a.accum + (size_t)m * a.N + n_out;
+                    if (!gated) {
+                        float total;
+                        if (accum_add(word, sum, a.splits, total)) {
+                            if constexpr (EXT) {
+                                finish_store(a.epi, a.D, m, n_out, total);
+                            } else if (a.epi.out_f32) {
+                                reinterpret_cast<float*>(a.D)[(size_t)m * a.N + n_out] = total;
+                            } else {
+                                reinterpret_cast<half_t*>(a.D)[(size_t)m * a.N + n_out] = (half_t)total;
+                            }
+                            accum_reset(word);
+                        }
+                    } else if (col_out < 64) {
+                        const float* usrc = src + 64;
+                        const float usum =
+                            (usrc[0] + usrc[32 * kRedStride]) + (usrc[64 * kRedStride] + usrc[96 * kRedStride]);
+                        float total_g, total_u;
+                        if (accum_add_pair(word, word + 64, sum, usum, a.splits, total_g, total_u)) {
+                            finish_store_gated(a.epi, a.D, m, 64 * strip + col_out, total_g, total_u);
+                            accum_reset(word);
                         }
                     }
                 }
@@ -488,10 +562,10 @@ static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_overr
     return p;
 }
 
-template <int MT>
+template <int MT, bool EXT>
 static hipError_t tile_launch_one(const TileArgs& a, int grid, hipStream_t stream) {
     const size_t shmem = TileLds<MT>::kBytes;
-    auto kern = &w4a16_tile_kernel<MT>;
+    auto kern = &w4a16_tile_kernel<MT, EXT>;
     if (shmem > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -503,8 +577,8 @@ static hipError_t tile_launch_one(const TileArgs& a, int grid, hipStream_t strea
 
 // tune: bits 0..7 force the number of K splits, bits 8..11 the number of 32-row M tiles per
 // workgroup (0 = choose)
-int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, void* accum, size_t accum_bytes,
-                int m, int n, int k, int groups, bool out_f32, unsigned tune, hipStream_t stream) {
+int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, const Epilogue& epi, void* accum,
+                size_t accum_bytes, int m, int n, int k, int groups, unsigned tune, hipStream_t stream) {
     const TilePlan plan = tile_plan(m, n, k, (int)(tune & 0xffu), (int)((tune >> 8) & 0xfu));
     if (plan.splits > 1 && (!accum || accum_bytes < (size_t)m * n * sizeof(unsigned long long)))
         return UNIQL_E_WORKSPACE;
@@ -523,13 +597,17 @@ int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* 
     a.gps = plan.gps;
     a.splits = plan.splits;
     a.mblocks = ceil_div_i(m, 32 * plan.mtiles);
-    a.out_f32 = out_f32 ? 1 : 0;
+    a.epi = epi;
     const int64_t grid = (int64_t)(n / 128) * a.mblocks * a.splits;
     if (grid > 0x7fffffffLL) return UNIQL_E_SHAPE;
     hipError_t e;
-    if (plan.mtiles == 1) e = tile_launch_one<1>(a, (int)grid, stream);
-    else if (plan.mtiles == 2) e = tile_launch_one<2>(a, (int)grid, stream);
-    else e = tile_launch_one<4>(a, (int)grid, stream);
+    const bool ext = epi.gated || epi.bias || epi.n_store != n || epi.ldd != n || !epi.vec_ok;
+    if (plan.mtiles == 1)
+        e = ext ? tile_launch_one<1, true>(a, (int)grid, stream) : tile_launch_one<1, false>(a, (int)grid, stream);
+    else if (plan.mtiles == 2)
+        e = ext ? tile_launch_one<2, true>(a, (int)grid, stream) : tile_launch_one<2, false>(a, (int)grid, stream);
+    else
+        e = ext ? tile_launch_one<4, true>(a, (int)grid, stream) : tile_launch_one<4, false>(a, (int)grid, stream);
     return e == hipSuccess ? UNIQL_OK : UNIQL_E_LAUNCH;
 }
 

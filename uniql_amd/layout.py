@@ -147,6 +147,33 @@ def quantize_and_pack(w: torch.Tensor, group_size: int = GROUP_SIZE, scale: torc
     return w_ref, pack_codes(codes), permute_scales(scale, kp, np_, group_size)
 
 
+# ---- fusing layers that read the same input ---------------------------------------------
+def concat_columns(weights, scales):
+    """Packed tensors of layers with the same K, side by side along N: the packed words and the
+    permuted scales of every 64-column block are contiguous, so this is a plain concatenation
+    (every width must be a multiple of 64; the module pads to 256)."""
+    for w, s in zip(weights, scales):
+        if s.shape[1] % CHUNK_N or w.shape[1] != 2 * s.shape[1]:
+            raise ValueError("every layer must be padded to a multiple of 64 columns")
+    return torch.cat(list(weights), dim=1).contiguous(), torch.cat(list(scales), dim=1).contiguous()
+
+
+def interleave_gate_up(gate_w, gate_s, up_w, up_s):
+    """Gate and up projection interleaved in blocks of 64 columns (block 2c = columns 64c.. of
+    gate, block 2c+1 = the same columns of up): the layout the kernels' silu(gate) * up
+    epilogue reads.  Returns (packed int32 [K/16, 4 Np], scale fp16 [G, 2 Np])."""
+    if gate_w.shape != up_w.shape or gate_s.shape != up_s.shape:
+        raise ValueError("gate and up projections must have the same shape")
+    rows, words = gate_w.shape
+    groups, n_pad = gate_s.shape
+    if n_pad % CHUNK_N or words != 2 * n_pad:
+        raise ValueError("projections must be padded to a multiple of 64 columns")
+    blocks = n_pad // CHUNK_N
+    w = torch.stack((gate_w.view(rows, blocks, 2 * CHUNK_N), up_w.view(rows, blocks, 2 * CHUNK_N)), dim=2)
+    s = torch.stack((gate_s.view(groups, blocks, CHUNK_N), up_s.view(groups, blocks, CHUNK_N)), dim=2)
+    return w.reshape(rows, 2 * words).contiguous(), s.reshape(groups, 2 * n_pad).contiguous()
+
+
 # ---- embedding table: one scale per row, 8 codes per word, nibble i <- element [0,2,4,6,1,3,5,7][i]
 def pack_embedding_codes(codes: torch.Tensor) -> torch.Tensor:
     """codes [V, D] in 0..15 -> int32 [V, D/8] (quant_embedding_layers.py:39-43)."""

@@ -16,8 +16,9 @@ import torch
 from . import _capi
 
 __all__ = [
-    "w4a16o16_gemm", "w4a16_gemm_ex", "w4a16_dequant", "w4a16_embedding_lookup",
+    "w4a16o16_gemm", "w4a16_gemm_ex", "w4a16_linear", "w4a16_dequant", "w4a16_embedding_lookup",
     "fast_hadamard_transform", "hadamard_blockwise", "unsupported_hadamard_variant",
+    "w4a16_quantize", "w4a16_pack", "w4a16_unpack", "w4_embedding_quantize", "rope_indices_",
 ]
 
 
@@ -95,6 +96,73 @@ def w4a16_gemm_ex(A: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: 
             size_m, size_n, size_k, groups, had_block, float(had_scale), flags, _stream_ptr(dev))
     _capi.check(code, "uniql_w4a16_gemm")
     return D
+
+
+def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: torch.Tensor, size_n: int,
+                 size_k: int, *, out_features: int | None = None, bias: torch.Tensor | None = None,
+                 silu_mul: bool = False, had_block: int = 0, had_scale: float = 1.0, out_f32: bool = False,
+                 out: torch.Tensor | None = None, flags: int = 0) -> torch.Tensor:
+    """The layer's whole forward in one call (uniql_w4a16_linear): x [m, in_features] with
+    in_features <= size_k (the kernel pads), product with the packed weights, only the first
+    `out_features` columns stored, `bias` added with the reference's rounding.  With
+    `silu_mul` the packed tensors hold a gate and an up projection interleaved in 64-column
+    blocks (layout.interleave_gate_up) and the result is silu(gate) * up, [m, out_features].
+    `out`: optional destination, a 2-D view with unit inner stride (for example a column range
+    of a larger buffer)."""
+    for t, name in ((x, "x"), (B, "B"), (s, "s"), (workspace, "workspace")):
+        _require_gpu(t, name)
+    if x.dtype != torch.float16 or s.dtype != torch.float16:
+        raise RuntimeError("x and s must be float16")
+    if B.dtype != torch.int32 or workspace.dtype != torch.int32:
+        raise RuntimeError("B and workspace must be int32")
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise RuntimeError("x must be 2-D with unit stride along K")
+    m, k_in = x.shape
+    if not (size_k - 128 < k_in <= size_k):
+        raise RuntimeError(f"x has {k_in} columns, the packed weights cover {size_k}")
+    if not (B.is_contiguous() and s.is_contiguous() and workspace.is_contiguous()):
+        raise RuntimeError("B, s and workspace must be contiguous")
+    if tuple(B.shape) != (size_k // 16, 2 * size_n) or s.dim() != 2 or s.shape[1] != size_n:
+        raise RuntimeError("B / s shapes do not match size_k, size_n")
+    n_max = size_n // 2 if silu_mul else size_n
+    n_out = n_max if out_features is None else int(out_features)
+    if not 0 < n_out <= n_max:
+        raise RuntimeError(f"out_features={n_out} does not fit the packed width {n_max}")
+    if bias is not None:
+        _require_gpu(bias, "bias")
+        if bias.dtype != torch.float16 or not bias.is_contiguous() or bias.numel() != (2 if silu_mul else 1) * n_out:
+            raise RuntimeError("bias must be contiguous float16 with one entry per output column")
+    if k_in % 8 or (m > 1 and x.stride(0) % 8) or x.data_ptr() % 16:
+        # rare: rows that cannot be read in 16-byte pieces are copied (and padded) here
+        x = torch.nn.functional.pad(x, (0, size_k - k_in))
+        k_in = size_k
+    lib = _capi.load()
+    dev = x.device
+    out_dtype = torch.float32 if out_f32 else torch.float16
+    with torch.cuda.device(dev):
+        if out is None:
+            out = torch.empty((m, n_out), dtype=out_dtype, device=dev)
+        elif out.dtype != out_dtype or tuple(out.shape) != (m, n_out) or out.stride(1) != 1 or out.device != dev:
+            raise RuntimeError("out must be a [m, out_features] view with unit inner stride on x's device")
+        if m == 0:
+            return out
+        need_acc = lib.uniql_w4a16_gemm_accum_bytes(m, size_n, size_k)
+        accum = _accumulator(dev, need_acc) if need_acc else None
+        need_tmp = lib.uniql_w4a16_linear_temp_bytes(m, size_n, size_k, k_in, had_block)
+        temp = torch.empty(need_tmp, dtype=torch.uint8, device=dev) if need_tmp else None
+        if out_f32:
+            flags |= _capi.F_OUT_F32
+        lda = x.stride(0) if m > 1 else max(k_in + (-k_in) % 8, 8)
+        ldd = out.stride(0) if m > 1 else n_out
+        code = lib.uniql_w4a16_linear(
+            x.data_ptr(), lda, k_in, B.data_ptr(), s.data_ptr(), bias.data_ptr() if bias is not None else None,
+            out.data_ptr(), ldd, n_out, _capi.EPI_SILU_MUL if silu_mul else _capi.EPI_NONE,
+            workspace.data_ptr(), workspace.numel(),
+            accum.data_ptr() if accum is not None else None, accum.numel() * 8 if accum is not None else 0,
+            temp.data_ptr() if temp is not None else None, need_tmp,
+            m, size_n, size_k, s.shape[0], had_block, float(had_scale), flags, _stream_ptr(dev))
+    _capi.check(code, "uniql_w4a16_linear")
+    return out
 
 
 def w4a16o16_gemm(A, B, s, workspace, size_m, size_n, size_k, output_transpose=False,
@@ -224,6 +292,68 @@ def w4a16_embedding_lookup(input: torch.Tensor, weight: torch.Tensor, scale: tor
                                              out.data_ptr(), vocab, dim, _stream_ptr(dev))
     _capi.check(code, "uniql_w4_embedding_lookup")
     return out
+
+
+def w4_embedding_quantize(weight: torch.Tensor):
+    """fp16 table [vocab, dim] on the GPU -> (packed int32 [vocab, dim/8], scales fp16 [vocab]) with the
+    arithmetic of W4O16Embedding.from_fp16 (quant_embedding_layers.py:26-48) bit for bit."""
+    _require_gpu(weight, "weight")
+    if weight.dtype != torch.float16 or weight.dim() != 2 or weight.stride(1) != 1:
+        raise RuntimeError("weight must be float16 [vocab, dim] with unit inner stride")
+    vocab, dim = weight.shape
+    if dim % 8 or weight.stride(0) % 8 or weight.data_ptr() % 16:
+        raise RuntimeError("embedding_dim and the row stride must be multiples of 8")
+    lib = _capi.load()
+    dev = weight.device
+    with torch.cuda.device(dev):
+        packed = torch.empty((vocab, dim // 8), dtype=torch.int32, device=dev)
+        scales = torch.empty(vocab, dtype=torch.float16, device=dev)
+        code = lib.uniql_w4_embedding_quantize(weight.data_ptr(), weight.stride(0) if vocab > 1 else dim,
+                                               packed.data_ptr(), scales.data_ptr(), vocab, dim, _stream_ptr(dev))
+    _capi.check(code, "uniql_w4_embedding_quantize")
+    return packed, scales
+
+
+def rope_indices_(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                  indices: torch.Tensor) -> None:
+    """In-place rotary embedding with gathered frequencies on token-major tensors:
+    q [batch, seq, n_q_heads, d], k [batch, seq, n_kv_heads, d] (last two axes contiguous, one row
+    stride over batch and seq), cos / sin [1 or batch, seq, D], indices [n_kv_heads, d]
+    (uint8, int32 or int64)."""
+    for t, name in ((q, "q"), (k, "k"), (cos, "cos"), (sin, "sin"), (indices, "indices")):
+        _require_gpu(t, name)
+    if not (q.dtype == k.dtype == cos.dtype == sin.dtype == torch.float16):
+        raise RuntimeError("q, k, cos and sin must be float16")
+    if q.dim() != 4 or k.dim() != 4 or cos.dim() != 3 or sin.shape != cos.shape:
+        raise RuntimeError("expected q, k [batch, seq, heads, d] and cos, sin [1 or batch, seq, D]")
+    batch, seq, n_qh, d = q.shape
+    n_kh = k.shape[2]
+    if k.shape[0] != batch or k.shape[1] != seq or k.shape[3] != d:
+        raise RuntimeError("q and k disagree on batch, sequence length or head width")
+    if tuple(indices.shape) != (n_kh, d):
+        raise RuntimeError(f"indices must be [{n_kh}, {d}]")
+    index_bytes = {torch.uint8: 1, torch.int32: 4, torch.int64: 8}.get(indices.dtype)
+    if index_bytes is None:
+        raise RuntimeError("indices must be uint8, int32 or int64")
+    if cos.shape[0] not in (1, batch) or cos.shape[1] != seq:
+        raise RuntimeError("cos / sin must cover [1 or batch, seq]")
+
+    def token_major(t, heads):
+        ok = t.stride(3) == 1 and t.stride(2) == d and (batch == 1 or t.stride(0) == seq * t.stride(1))
+        if not ok:
+            raise RuntimeError("q / k must be token-major with contiguous heads (use .contiguous())")
+        return t.stride(1) if seq > 1 else (t.stride(0) if batch > 1 else heads * d)
+
+    q_stride, k_stride = token_major(q, n_qh), token_major(k, n_kh)
+    if not (cos.is_contiguous() and sin.is_contiguous() and indices.is_contiguous()):
+        raise RuntimeError("cos, sin and indices must be contiguous")
+    lib = _capi.load()
+    dev = q.device
+    with torch.cuda.device(dev):
+        code = lib.uniql_rope_indices(q.data_ptr(), q_stride, k.data_ptr(), k_stride, cos.data_ptr(), sin.data_ptr(),
+                                      cos.shape[2], indices.data_ptr(), index_bytes, batch * seq, seq, cos.shape[0],
+                                      n_qh, n_kh, d, cos.shape[2], _stream_ptr(dev))
+    _capi.check(code, "uniql_rope_indices")
 
 
 def hadamard_blockwise(x: torch.Tensor, scale: float, block: int | None = None) -> torch.Tensor:

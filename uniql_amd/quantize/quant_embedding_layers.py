@@ -26,7 +26,11 @@ class W4O16Embedding(nn.Module):
     def from_fp16(cls, originalLayer: nn.Embedding):
         w = originalLayer.weight.data
         q = cls(originalLayer.num_embeddings, originalLayer.embedding_dim, device=w.device)
-        packed, scales = layout.quantize_embedding(w)
+        if w.is_cuda and w.dtype == torch.float16 and originalLayer.embedding_dim % 8 == 0:
+            # the device kernel: same codes and scales bit for bit, no host round trip
+            packed, scales = ops.w4_embedding_quantize(w.contiguous())
+        else:
+            packed, scales = layout.quantize_embedding(w)
         q.scales = scales.to(w.device)
         q.weight.data = packed.to(w.device)
         return q

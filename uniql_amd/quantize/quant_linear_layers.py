@@ -96,22 +96,16 @@ class W4A16B16O16Linear(nn.Module):
 
     @torch.no_grad()
     def forward(self, x):
+        """Padding of the input, the product, the cut of the padded output columns and the bias
+        (quant_linear_layers.py:92-114) happen inside one kernel call."""
         lead = x.shape[:-1]
         x2 = x.reshape(-1, x.shape[-1])
-        if not x2.is_contiguous():
+        if x2.stride(-1) != 1:
             x2 = x2.contiguous()
-        if self.pad_in:
-            x2 = F.pad(x2, (0, self.pad_in))
-        if self.had_block:
-            y = ops.w4a16_gemm_ex(x2, self.weight, self.scale, self.workspace, x2.shape[0], self.size_n,
-                                  self.size_k, had_block=self.had_block, had_scale=self.had_scale)
-        else:
-            y = ops.w4a16o16_gemm(x2, self.weight, self.scale, self.workspace, x2.shape[0], self.size_n,
-                                  self.size_k, False, -1, -1, -1, self.max_par)
-        if self.pad_out:
-            y = y[:, :self.out_features]
-        y = y.reshape(*lead, self.out_features)
-        return y if self.bias is None else y + self.bias
+        y = ops.w4a16_linear(x2, self.weight, self.scale, self.workspace, self.size_n, self.size_k,
+                             out_features=self.out_features, bias=None if self.bias is None else self.bias.data,
+                             had_block=self.had_block, had_scale=self.had_scale)
+        return y.view(*lead, self.out_features)
 
     def __repr__(self):
         return (f"W4A16B16O16Linear(in_features={self.in_features}, out_features={self.out_features}, "
