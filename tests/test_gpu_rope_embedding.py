@@ -17,7 +17,10 @@ def pruned_indices(hk, d, D, seed):
 
 
 @pytest.mark.parametrize("b,hq,hk,s,d,D", [(1, 32, 8, 1, 128, 128), (2, 32, 8, 17, 108, 128), (1, 4, 4, 33, 64, 64),
-                                           (3, 6, 2, 5, 14, 32), (1, 32, 8, 1024, 108, 128), (2, 28, 4, 9, 6, 128)])
+                                           (3, 6, 2, 5, 14, 32), (1, 32, 8, 1024, 108, 128), (2, 28, 4, 9, 6, 128),
+                                           # 64 rows and more take the kernel that builds the gathered table in LDS
+                                           (1, 32, 8, 100, 128, 128), (2, 32, 32, 40, 64, 128), (4, 6, 2, 20, 14, 32),
+                                           (1, 16, 2, 64, 96, 256)])
 @pytest.mark.parametrize("index_dtype", [torch.uint8, torch.int64, torch.int32])
 def test_rope_indices_bit_exact(gpu, b, hq, hk, s, d, D, index_dtype):
     from uniql_amd import ops

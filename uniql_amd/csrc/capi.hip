@@ -19,7 +19,7 @@ int embedding_quantize_launch(const void* W, int64_t ldw, void* packed, void* sc
                               hipStream_t stream);
 int rope_indices_launch(void* q, int64_t q_row_stride, void* k, int64_t k_row_stride, const void* cos, const void* sin,
                         int64_t cos_row_stride, const void* indices, int index_bytes, int64_t rows, int seq_len,
-                        int cos_batch, int n_qh, int n_kh, int hd, hipStream_t stream);
+                        int cos_batch, int n_qh, int n_kh, int hd, int cos_dim, hipStream_t stream);
 int fwht_launch(const void* x, void* y, int64_t rows, int dim, int block, float scale, int dtype,
                 hipStream_t stream);
 int quantize_launch(const void* W, int64_t ldw, const void* given_scales, void* B, void* S, int out_features,
@@ -227,7 +227,7 @@ int uniql_rope_indices(void* q, int64_t q_row_stride, void* k, int64_t k_row_str
     if (rows == 0) return UNIQL_OK;
     if (!q || !k || !cos || !sin || !indices) return UNIQL_E_NULL;
     return rope_indices_launch(q, q_row_stride, k, k_row_stride, cos, sin, cos_row_stride, indices, index_bytes,
-                               rows, seq_len, cos_batch, n_q_heads, n_kv_heads, head_dim,
+                               rows, seq_len, cos_batch, n_q_heads, n_kv_heads, head_dim, cos_dim,
                                reinterpret_cast<hipStream_t>(stream));
 }
 

@@ -3,9 +3,10 @@
 // key/value head, the list of the original columns they retained; column j of such a head is
 // rotated with the frequency of original column indices[head][j].
 //
-// One thread rotates two neighbouring column pairs (j, j + d/2), (j+1, j+1 + d/2) of one head of
-// one token: 4-byte loads and stores, consecutive lanes on consecutive columns.  Every value is
-// read once and written once; cos / sin rows are shared by all heads of a token and stay in cache.
+// One thread rotates up to eight neighbouring column pairs (j, j + d/2) of one head of one token
+// with 16-byte loads and stores (4- or 2-byte ones when the head width does not allow more),
+// consecutive lanes on consecutive columns.  Every value is read once and written once; cos /
+// sin rows are shared by all heads of a token and stay in cache.
 //
 // Arithmetic: out = x * cos_g + rotate_half(x) * sin_g with both products and the sum rounded to
 // fp16 one after the other, which is what the tensor expression of the reference computes on
@@ -21,7 +22,6 @@ struct RopeArgs {
     const half_t* sin;
     const void* indices;  // [n_kh][hd], index_bytes wide
     int64_t q_row_stride, k_row_stride, cos_row_stride;
-    int64_t work;         // rows * (n_qh + n_kh) * (hd / 2 / VEC)
     int seq_len, cos_batch, n_qh, n_kh, hd, index_bytes;
 };
 
@@ -43,16 +43,29 @@ __device__ __forceinline__ void rotate_pair(half_t& lo, half_t& hi, half_t c_lo,
     hi = (half_t)((float)a_hi + (float)r_hi);
 }
 
-template <int VEC>  // columns per thread and half: 2 (4-byte accesses) or 1
+template <int VEC>
+struct HalfVec;  // VEC fp16 values moved with one access
+template <>
+struct HalfVec<8> { typedef h8 type; };
+template <>
+struct HalfVec<2> { typedef h2 type; };
+template <>
+struct HalfVec<1> { typedef half_t type; };
+
+// VEC columns per thread and half of the head: 8 (16-byte accesses), 2 or 1.  A block covers
+// 256 consecutive work items of one token, so the only divisions are 32-bit ones.
+template <int VEC>
 __global__ __launch_bounds__(256) void rope_indices_kernel(const RopeArgs a) {
-    const int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= a.work) return;
+    typedef typename HalfVec<VEC>::type vec_t;
     const int half = a.hd >> 1;
     const int per_head = half / VEC;
-    const int heads = a.n_qh + a.n_kh;
-    const int j = (int)(idx % per_head) * VEC;
-    const int head = (int)((idx / per_head) % heads);
-    const int64_t row = idx / ((int64_t)per_head * heads);
+    const int per_row = (a.n_qh + a.n_kh) * per_head;
+    const int blocks_per_row = (per_row + 255) >> 8;
+    const int64_t row = blockIdx.x / blocks_per_row;
+    const int t = (int)(blockIdx.x % blocks_per_row) * 256 + threadIdx.x;
+    if (t >= per_row) return;
+    const int head = t / per_head;
+    const int j = (t - head * per_head) * VEC;
 
     const bool is_q = head < a.n_qh;
     const int kv_head = is_q ? head / (a.n_qh / a.n_kh) : head - a.n_qh;
@@ -62,16 +75,17 @@ __global__ __launch_bounds__(256) void rope_indices_kernel(const RopeArgs a) {
     const half_t* cos_row = a.cos + table_row * a.cos_row_stride;
     const half_t* sin_row = a.sin + table_row * a.cos_row_stride;
 
+    vec_t lo_v = *reinterpret_cast<const vec_t*>(x + j), hi_v = *reinterpret_cast<const vec_t*>(x + half + j);
     half_t lo[VEC], hi[VEC];
-    if (VEC == 2) {
-        const h2 l = *reinterpret_cast<const h2*>(x + j), h = *reinterpret_cast<const h2*>(x + half + j);
-        lo[0] = l.x;
-        lo[VEC - 1] = l.y;
-        hi[0] = h.x;
-        hi[VEC - 1] = h.y;
+    if constexpr (VEC == 1) {
+        lo[0] = lo_v;
+        hi[0] = hi_v;
     } else {
-        lo[0] = x[j];
-        hi[0] = x[half + j];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+            lo[v] = lo_v[v];
+            hi[v] = hi_v[v];
+        }
     }
 #pragma unroll
     for (int v = 0; v < VEC; ++v) {
@@ -79,18 +93,90 @@ __global__ __launch_bounds__(256) void rope_indices_kernel(const RopeArgs a) {
         const int i_hi = load_index(a.indices, a.index_bytes, kv_head * a.hd + half + j + v);
         rotate_pair(lo[v], hi[v], cos_row[i_lo], sin_row[i_lo], cos_row[i_hi], sin_row[i_hi]);
     }
-    if (VEC == 2) {
-        *reinterpret_cast<h2*>(x + j) = h2{lo[0], lo[VEC - 1]};
-        *reinterpret_cast<h2*>(x + half + j) = h2{hi[0], hi[VEC - 1]};
+    if constexpr (VEC == 1) {
+        lo_v = lo[0];
+        hi_v = hi[0];
     } else {
-        x[j] = lo[0];
-        x[half + j] = hi[0];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+            lo_v[v] = lo[v];
+            hi_v[v] = hi[v];
+        }
+    }
+    *reinterpret_cast<vec_t*>(x + j) = lo_v;
+    *reinterpret_cast<vec_t*>(x + half + j) = hi_v;
+}
+
+// Many tokens: one workgroup per token builds the token's gathered (cos, sin) pairs once per
+// key/value head in LDS (n_kv_heads x head_dim entries of 4 bytes) and every query head of the
+// group reads them from there, instead of every element gathering from the tables in memory.
+template <int VEC>
+__global__ __launch_bounds__(256) void rope_indices_lds_kernel(const RopeArgs a, int cos_dim) {
+    typedef typename HalfVec<VEC>::type vec_t;
+    extern __shared__ __attribute__((aligned(16))) uint32_t rope_lds[];
+    uint16_t* trow = reinterpret_cast<uint16_t*>(rope_lds);  // the token's cos row, then its sin row
+    uint32_t* tab = rope_lds + ((cos_dim + 3) & ~3);         // entry (kv head, column): cos | sin << 16
+    const int tid = threadIdx.x;
+    const int64_t row = blockIdx.x;
+    const int64_t table_row = a.cos_batch == 1 ? row % a.seq_len : row;
+    const uint16_t* cos_row = reinterpret_cast<const uint16_t*>(a.cos + table_row * a.cos_row_stride);
+    const uint16_t* sin_row = reinterpret_cast<const uint16_t*>(a.sin + table_row * a.cos_row_stride);
+    for (int i = tid; i < cos_dim; i += 256) {
+        trow[i] = cos_row[i];
+        trow[cos_dim + i] = sin_row[i];
+    }
+    __syncthreads();
+    const int entries = a.n_kh * a.hd;
+    for (int e = tid; e < entries; e += 256) {
+        const int i = load_index(a.indices, a.index_bytes, e);
+        tab[e] = (uint32_t)trow[i] | ((uint32_t)trow[cos_dim + i] << 16);
+    }
+    __syncthreads();
+    const int half = a.hd >> 1;
+    const int per_head = half / VEC;
+    const int per_row = (a.n_qh + a.n_kh) * per_head;
+    for (int t = tid; t < per_row; t += 256) {
+        const int head = t / per_head;
+        const int j = (t - head * per_head) * VEC;
+        const bool is_q = head < a.n_qh;
+        const int kv_head = is_q ? head / (a.n_qh / a.n_kh) : head - a.n_qh;
+        half_t* x = is_q ? a.q + row * a.q_row_stride + (int64_t)head * a.hd
+                         : a.k + row * a.k_row_stride + (int64_t)(head - a.n_qh) * a.hd;
+        vec_t lo_v = *reinterpret_cast<const vec_t*>(x + j), hi_v = *reinterpret_cast<const vec_t*>(x + half + j);
+        const uint32_t* e_lo = tab + kv_head * a.hd + j;
+        const uint32_t* e_hi = e_lo + half;
+#pragma unroll
+        for (int v = 0; v < VEC; ++v) {
+            const uint32_t w_lo = e_lo[v], w_hi = e_hi[v];
+            const half_t c_lo = __builtin_bit_cast(half_t, (uint16_t)(w_lo & 0xffffu));
+            const half_t s_lo = __builtin_bit_cast(half_t, (uint16_t)(w_lo >> 16));
+            const half_t c_hi = __builtin_bit_cast(half_t, (uint16_t)(w_hi & 0xffffu));
+            const half_t s_hi = __builtin_bit_cast(half_t, (uint16_t)(w_hi >> 16));
+            half_t lo, hi;
+            if constexpr (VEC == 1) {
+                lo = lo_v;
+                hi = hi_v;
+            } else {
+                lo = lo_v[v];
+                hi = hi_v[v];
+            }
+            rotate_pair(lo, hi, c_lo, s_lo, c_hi, s_hi);
+            if constexpr (VEC == 1) {
+                lo_v = lo;
+                hi_v = hi;
+            } else {
+                lo_v[v] = lo;
+                hi_v[v] = hi;
+            }
+        }
+        *reinterpret_cast<vec_t*>(x + j) = lo_v;
+        *reinterpret_cast<vec_t*>(x + half + j) = hi_v;
     }
 }
 
 int rope_indices_launch(void* q, int64_t q_row_stride, void* k, int64_t k_row_stride, const void* cos, const void* sin,
                         int64_t cos_row_stride, const void* indices, int index_bytes, int64_t rows, int seq_len,
-                        int cos_batch, int n_qh, int n_kh, int hd, hipStream_t stream) {
+                        int cos_batch, int n_qh, int n_kh, int hd, int cos_dim, hipStream_t stream) {
     RopeArgs a;
     a.q = reinterpret_cast<half_t*>(q);
     a.k = reinterpret_cast<half_t*>(k);
@@ -106,16 +192,33 @@ int rope_indices_launch(void* q, int64_t q_row_stride, void* k, int64_t k_row_st
     a.n_kh = n_kh;
     a.hd = hd;
     a.index_bytes = index_bytes;
+    if (rows == 0) return UNIQL_OK;
     const int half = hd / 2;
-    // 4-byte accesses need even offsets everywhere
-    const bool vec2 = half % 2 == 0 && q_row_stride % 2 == 0 && k_row_stride % 2 == 0 &&
-                      (reinterpret_cast<uintptr_t>(q) & 3u) == 0 && (reinterpret_cast<uintptr_t>(k) & 3u) == 0;
-    const int vec = vec2 ? 2 : 1;
-    a.work = rows * (int64_t)(n_qh + n_kh) * (half / vec);
-    if (a.work == 0) return UNIQL_OK;
-    const int64_t blocks = (a.work + 255) / 256;
+    // the widest access every offset (head start, half-head start, row start) is aligned for
+    const uintptr_t bases = reinterpret_cast<uintptr_t>(q) | reinterpret_cast<uintptr_t>(k);
+    int vec = 1;
+    if (half % 8 == 0 && q_row_stride % 8 == 0 && k_row_stride % 8 == 0 && (bases & 15u) == 0) vec = 8;
+    else if (half % 2 == 0 && q_row_stride % 2 == 0 && k_row_stride % 2 == 0 && (bases & 3u) == 0) vec = 2;
+    // enough tokens to fill the chip with one workgroup each, and tables that fit LDS
+    const size_t lds_bytes = ((size_t)((cos_dim + 3) & ~3) + (size_t)n_kh * hd) * 4;
+    if (rows >= 64 && lds_bytes <= 32 * 1024 && rows <= 0x7fffffffLL) {
+        if (vec == 8)
+            hipLaunchKernelGGL(rope_indices_lds_kernel<8>, dim3((unsigned)rows), dim3(256), lds_bytes, stream, a, cos_dim);
+        else if (vec == 2)
+            hipLaunchKernelGGL(rope_indices_lds_kernel<2>, dim3((unsigned)rows), dim3(256), lds_bytes, stream, a, cos_dim);
+        else
+            hipLaunchKernelGGL(rope_indices_lds_kernel<1>, dim3((unsigned)rows), dim3(256), lds_bytes, stream, a, cos_dim);
+        return hipGetLastError() == hipSuccess ? UNIQL_OK : UNIQL_E_LAUNCH;
+    }
+    // few tokens: the direct gather, narrow accesses (more threads in flight hide the dependent
+    // index -> table loads better than wide accesses do)
+    if (vec == 8) vec = 2;
+    const int per_row = (n_qh + n_kh) * (half / vec);
+    const int64_t blocks = rows * ((per_row + 255) / 256);
     if (blocks > 0x7fffffffLL) return UNIQL_E_SHAPE;
-    if (vec2)
+    if (vec == 8)
+        hipLaunchKernelGGL(rope_indices_kernel<8>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
+    else if (vec == 2)
         hipLaunchKernelGGL(rope_indices_kernel<2>, dim3((unsigned)blocks), dim3(256), 0, stream, a);
     else
         hipLaunchKernelGGL(rope_indices_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, stream, a);

@@ -74,6 +74,13 @@ __device__ __forceinline__ void store_eight(const Epilogue& e, void* D, int m, i
             *reinterpret_cast<f4*>(d + 4) = hi;
             return;
         }
+        if (!e.out_f32 && !e.bias) {
+            const h2 r0 = h2{(half_t)lo[0], (half_t)lo[1]}, r1 = h2{(half_t)lo[2], (half_t)lo[3]};
+            const h2 r2 = h2{(half_t)hi[0], (half_t)hi[1]}, r3 = h2{(half_t)hi[2], (half_t)hi[3]};
+            *reinterpret_cast<u32x4*>(reinterpret_cast<half_t*>(D) + o) =
+                u32x4{h2_to_bits(r0), h2_to_bits(r1), h2_to_bits(r2), h2_to_bits(r3)};
+            return;
+        }
         if (!e.out_f32) {
             half_t r[8];
 #pragma unroll
