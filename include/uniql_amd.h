@@ -37,7 +37,11 @@ enum {
     UNIQL_F_OUT_F32 = 1 << 0,      /* D is float32 [m, n] instead of fp16 (test hook: the value before the final rounding) */
     UNIQL_F_FORCE_SKINNY = 1 << 1, /* use the weight-streaming kernel (default for m <= 16) whatever m is */
     UNIQL_F_FORCE_TILED = 1 << 2,  /* use the tiled MFMA kernel (default for m > 16) whatever m is */
-    UNIQL_F_TRANSPOSE_OUT = 1 << 3 /* reference's output_transpose; rejected with UNIQL_E_UNSUPPORTED */
+    UNIQL_F_TRANSPOSE_OUT = 1 << 3 /* the reference's output_transpose ("sequence length last",
+                                      csrc/linear/marlin_gemm_kernel.cuh:574-606,1023-1026): D is [n, ldd]
+                                      with D[j, i] = product[i, j]; uniql_w4a16_gemm uses ldd = m rounded up
+                                      to a multiple of 8 as the reference does and leaves the padding columns
+                                      untouched; uniql_w4a16_linear takes ldd >= m from the caller */
     /* tuning hooks, 0 = choose.  Streaming kernel: bits 8..15 K-groups per wavefront,
        bits 16..20 wavefronts per workgroup (4 or 8).
        Tiled kernel: bits 8..15 number of K splits over workgroups, bits 16..19 row tiles of 32

@@ -55,9 +55,40 @@ def test_argument_checks_need_no_gpu(lib):
     assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 1, 4096 + 64, 4096, 32, 0, 1.0, 0, None) == -2
     assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 1, 4096, 4096 + 16, 32, 0, 1.0, 0, None) == -2
     assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 1, 4096, 4096, 7, 0, 1.0, 0, None) == -2
-    assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 1, 4096, 4096, 32, 0, 1.0, 8, None) == -5
+    assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 1, 4096, 4096, 32, 0, 1.0, 8, None) == -1
     assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 1, 4096, 4096, 32, 0, 1.0, 0, None) == -1
     assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 0, 4096, 4096, 32, 0, 1.0, 0, None) == 0
+    g = lib.uniql_w4a16_linear
+    args = dict(A=None, lda=4096, k_in=4096, B=None, S=None, bias=None, D=None, ldd=4096, n_out=4096, epilogue=0,
+                workspace=None, workspace_len=0, accum=None, accum_bytes=0, temp=None, temp_bytes=0, m=1, n=4096,
+                k=4096, groups=32, had_block=0, had_scale=1.0, flags=0, stream=None)
+
+    def call(**kw):
+        return g(*{**args, **kw}.values())
+
+    assert call() == -1                                  # shapes fine, pointers missing
+    assert call(k_in=4096 - 128) == -2                   # a whole group of the input missing
+    assert call(k_in=4095) == -2                         # not a multiple of 8
+    assert call(n_out=4097) == -2
+    assert call(epilogue=1, n_out=2049) == -2            # a gated call stores at most n/2 columns
+    assert call(epilogue=1, n_out=2048, ldd=2048) == -1
+    assert call(epilogue=2) == -5
+    assert call(ldd=4095) == -2
+    assert call(flags=8, ldd=0) == -2                    # transposed: ldd counts rows
+    assert call(m=0) == 0
+    assert lib.uniql_w4a16_linear_temp_bytes(3, 4096, 4096, 4000, 0) == 3 * 4096 * 2
+    assert lib.uniql_w4a16_linear_temp_bytes(3, 4096, 4096, 4096, 0) == 0
+    r = lib.uniql_rope_indices
+    assert r(None, 4096, None, 1024, None, None, 128, None, 1, 4, 4, 1, 32, 8, 128, 128, None) == -1
+    assert r(None, 4096, None, 1024, None, None, 128, None, 2, 4, 4, 1, 32, 8, 128, 128, None) == -5
+    assert r(None, 4096, None, 1024, None, None, 128, None, 1, 4, 4, 1, 32, 5, 128, 128, None) == -2
+    assert r(None, 4096, None, 1024, None, None, 128, None, 1, 5, 4, 1, 32, 8, 128, 128, None) == -2
+    assert r(None, 4096, None, 1024, None, None, 128, None, 1, 4, 4, 1, 32, 8, 127, 128, None) == -2
+    assert r(None, 4095, None, 1024, None, None, 128, None, 1, 4, 4, 1, 32, 8, 128, 128, None) == -2
+    assert r(None, 4096, None, 1024, None, None, 128, None, 1, 0, 4, 1, 32, 8, 128, 128, None) == 0
+    assert lib.uniql_w4_embedding_quantize(None, 64, None, None, 10, 60, None) == -2
+    assert lib.uniql_w4_embedding_quantize(None, 64, None, None, 10, 64, None) == -1
+    assert lib.uniql_w4_embedding_quantize(None, 64, None, None, 0, 64, None) == 0
     assert lib.uniql_fwht(None, None, 4, 96, 96, 1.0, 0, None) == -2
     assert lib.uniql_fwht(None, None, 4, 128, 128, 1.0, 7, None) == -5
     assert lib.uniql_w4_embedding_lookup(None, 5, None, None, None, 10, 12, None) == -2

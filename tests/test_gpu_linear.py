@@ -204,14 +204,28 @@ def test_full_width_hadamard_prologue(gpu, m):
     check_fp32_result(y32, p, ref, m, x=xr)
 
 
+@pytest.mark.parametrize("m", [1, 5, 16, 40, 130])
+def test_output_transpose(gpu, m):
+    """the reference's output_transpose: D[n, m8], row index last, m rounded up to 8"""
+    from uniql_amd import ops
+    k, n = 512, 384
+    p = make_linear_problem(m, k, n, seed=m)
+    x, b, s = to_gpu(p, gpu)
+    ws = workspace_for(n, gpu)
+    want = ops.w4a16o16_gemm(x, b, s, ws, m, n, k)
+    got = ops.w4a16o16_gemm(x, b, s, ws, m, n, k, True)
+    m8 = (m + 7) // 8 * 8
+    assert tuple(got.shape) == (n, m8)
+    assert torch.equal(got[:, :m], want.t())
+    assert int(got[:, m:].abs().sum()) == 0
+
+
 # ------------------------------------------------------------------ error paths
 def test_errors(gpu):
     from uniql_amd import ops
     p = make_linear_problem(1, 256, 256)
     x, b, s = to_gpu(p, gpu)
     ws = workspace_for(256, gpu)
-    with pytest.raises(RuntimeError):
-        ops.w4a16o16_gemm(x, b, s, ws, 1, 256, 256, True)                 # output_transpose
     with pytest.raises(RuntimeError):
         ops.w4a16o16_gemm(x, b, s, ws[:2], 1, 256, 256, False, -1, -1, -1, 16)   # workspace too small
     with pytest.raises(RuntimeError):

@@ -86,11 +86,11 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
                        int n, int k, int groups, int had_block, float had_scale, unsigned flags, void* stream) {
     const int rc = check_linear_shape(m, n, k, groups);
     if (rc != UNIQL_OK) return rc;
-    if (flags & UNIQL_F_TRANSPOSE_OUT) return UNIQL_E_UNSUPPORTED;
+    const bool transpose = (flags & UNIQL_F_TRANSPOSE_OUT) != 0;
     if (epilogue != UNIQL_EPI_NONE && epilogue != UNIQL_EPI_SILU_MUL) return UNIQL_E_UNSUPPORTED;
     const bool gated = epilogue == UNIQL_EPI_SILU_MUL;
     if (k_in <= 0 || k_in > k || k - k_in >= 128 || (k_in % 8) != 0) return UNIQL_E_SHAPE;
-    if (n_out <= 0 || n_out > (gated ? n / 2 : n) || ldd < n_out) return UNIQL_E_SHAPE;
+    if (n_out <= 0 || n_out > (gated ? n / 2 : n) || ldd < (transpose ? m : n_out)) return UNIQL_E_SHAPE;
     if (m == 0) return UNIQL_OK;
     if (!A || !B || !S || !D) return UNIQL_E_NULL;
     if (lda < k_in || (lda % 8) != 0) return UNIQL_E_ALIGN;
@@ -149,7 +149,8 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
     epi.n_store = n_out;
     epi.gated = gated ? 1 : 0;
     epi.out_f32 = out_f32 ? 1 : 0;
-    epi.vec_ok = (ldd % 8 == 0 && aligned16(D)) ? 1 : 0;
+    epi.transpose = transpose ? 1 : 0;
+    epi.vec_ok = (!transpose && ldd % 8 == 0 && aligned16(D)) ? 1 : 0;
     const unsigned tune = flags >> 8;  // tuning fields, see the header
     if (use_stream)
         return stream_launch(Ain, ld, k_valid, B, S, D, epi, accum, m, n, k, groups, had128, had_scale, tune, st);
@@ -160,7 +161,10 @@ int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, v
                      int64_t workspace_len, void* accum, size_t accum_bytes, void* temp, size_t temp_bytes, int m,
                      int n, int k, int groups, int had_block, float had_scale, unsigned flags, void* stream) {
     if (D && !aligned16(D)) return UNIQL_E_ALIGN;
-    return uniql_w4a16_linear(A, lda, k, B, S, nullptr, D, n, n, UNIQL_EPI_NONE, workspace, workspace_len, accum,
+    // transposed: D is [n, m8] with m8 = m rounded up to 8, as the reference allocates it
+    // (marlin_gemm_kernel.cuh:1023-1026)
+    const int64_t ldd = (flags & UNIQL_F_TRANSPOSE_OUT) ? (int64_t)((m + 7) / 8) * 8 : n;
+    return uniql_w4a16_linear(A, lda, k, B, S, nullptr, D, ldd, n, UNIQL_EPI_NONE, workspace, workspace_len, accum,
                               accum_bytes, temp, temp_bytes, m, n, k, groups, had_block, had_scale, flags, stream);
 }
 

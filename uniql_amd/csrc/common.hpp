@@ -92,6 +92,12 @@ struct Epilogue {
                          //    of output column 64 strip + c; the output is silu(gate) * up
     int out_f32;         // D is float32 and receives the values before any rounding
     int vec_ok;          // ldd and D allow 16-byte stores of eight fp16 outputs
+    int transpose;       // 1: D is [n_store][ldd] with the row index running along the inner axis
+                         //    (the reference's output_transpose, "sequence length last")
+
+    __device__ __forceinline__ size_t offset(int m, int n) const {
+        return transpose ? (size_t)n * ldd + m : (size_t)m * ldd + n;
+    }
 };
 
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
@@ -112,7 +118,7 @@ __device__ __forceinline__ half_t finish_half_gated(const Epilogue& e, int n, fl
 
 __device__ __forceinline__ void finish_store(const Epilogue& e, void* D, int m, int n, float v) {
     if (n >= e.n_store) return;
-    const size_t o = (size_t)m * e.ldd + n;
+    const size_t o = e.offset(m, n);
     if (e.out_f32)
         reinterpret_cast<float*>(D)[o] = e.bias ? v + (float)e.bias[n] : v;
     else
@@ -121,7 +127,7 @@ __device__ __forceinline__ void finish_store(const Epilogue& e, void* D, int m, 
 
 __device__ __forceinline__ void finish_store_gated(const Epilogue& e, void* D, int m, int n, float g, float u) {
     if (n >= e.n_store) return;
-    const size_t o = (size_t)m * e.ldd + n;
+    const size_t o = e.offset(m, n);
     if (e.out_f32) {
         if (e.bias) {
             g += (float)e.bias[n];

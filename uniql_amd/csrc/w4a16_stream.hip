@@ -437,7 +437,7 @@ static hipError_t launch_waves(const StreamArgs& a, int waves, bool ext, hipStre
 template <bool HAD>
 static hipError_t launch_rows(const StreamArgs& a, int mt, int waves, hipStream_t stream) {
     const Epilogue& e = a.epi;
-    const bool ext = e.gated || e.bias || e.n_store != a.N || e.ldd != a.N || a.k_valid != a.K;
+    const bool ext = e.gated || e.bias || e.transpose || e.n_store != a.N || e.ldd != a.N || a.k_valid != a.K;
     if (mt == 4) return launch_waves<4, 16, HAD>(a, waves, ext, stream);
     if (mt == 2) return launch_waves<2, 16, HAD>(a, waves, ext, stream);
     if (a.M == 1) return launch_waves<1, 1, HAD>(a, waves, ext, stream);
@@ -477,7 +477,7 @@ int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const 
         a.M = mm;
         a.xrows = mt == 1 ? ((mm + 3) / 4) * 4 : mt * 16;
         a.X = reinterpret_cast<const half_t*>(A) + (size_t)m0 * lda;
-        a.D = reinterpret_cast<char*>(D) + (size_t)m0 * epi.ldd * out_elt;
+        a.D = reinterpret_cast<char*>(D) + (size_t)m0 * (epi.transpose ? 1 : epi.ldd) * out_elt;
         const hipError_t e = had128 ? launch_rows<true>(a, mt, plan.waves, stream)
                                     : launch_rows<false>(a, mt, plan.waves, stream);
         if (e != hipSuccess) return UNIQL_E_LAUNCH;

@@ -608,7 +608,7 @@ int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* 
     const int64_t grid = (int64_t)(n / 128) * a.mblocks * a.splits;
     if (grid > 0x7fffffffLL) return UNIQL_E_SHAPE;
     hipError_t e;
-    const bool ext = epi.gated || epi.bias || epi.n_store != n || epi.ldd != n || !epi.vec_ok;
+    const bool ext = epi.gated || epi.bias || epi.transpose || epi.n_store != n || epi.ldd != n || !epi.vec_ok;
     if (plan.mtiles == 1)
         e = ext ? tile_launch_one<1, true>(a, (int)grid, stream) : tile_launch_one<1, false>(a, (int)grid, stream);
     else if (plan.mtiles == 2)

@@ -54,8 +54,11 @@ def _require_gpu(t: torch.Tensor, name: str) -> None:
 
 def w4a16_gemm_ex(A: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: torch.Tensor,
                   size_m: int, size_n: int, size_k: int, *, had_block: int = 0,
-                  had_scale: float = 1.0, out_f32: bool = False, flags: int = 0) -> torch.Tensor:
-    """D[m, n] = rotate(A)[m, k] . dequant(B)[k, n].  `had_block` 0 means no rotation."""
+                  had_scale: float = 1.0, out_f32: bool = False, transpose_out: bool = False,
+                  flags: int = 0) -> torch.Tensor:
+    """D[m, n] = rotate(A)[m, k] . dequant(B)[k, n].  `had_block` 0 means no rotation.
+    transpose_out: the result comes as [n, m8] with m8 = m rounded up to 8 (the reference's
+    output_transpose layout, marlin_gemm_kernel.cuh:1023-1026); columns m.. are zero."""
     for t, name in ((A, "A"), (B, "B"), (s, "s"), (workspace, "workspace")):
         _require_gpu(t, name)
     if A.dtype != torch.float16 or s.dtype != torch.float16:
@@ -80,7 +83,11 @@ def w4a16_gemm_ex(A: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: 
     dev = A.device
     out_dtype = torch.float32 if out_f32 else torch.float16
     with torch.cuda.device(dev):
-        D = torch.empty((size_m, size_n), dtype=out_dtype, device=dev)
+        if transpose_out:
+            D = torch.zeros((size_n, (size_m + 7) // 8 * 8), dtype=out_dtype, device=dev)
+            flags |= _capi.F_TRANSPOSE_OUT
+        else:
+            D = torch.empty((size_m, size_n), dtype=out_dtype, device=dev)
         need_acc = lib.uniql_w4a16_gemm_accum_bytes(size_m, size_n, size_k)
         accum = _accumulator(dev, need_acc) if need_acc else None
         need_tmp = lib.uniql_w4a16_gemm_temp_bytes(size_m, size_n, size_k, had_block)
@@ -170,11 +177,10 @@ def w4a16o16_gemm(A, B, s, workspace, size_m, size_n, size_k, output_transpose=F
     """Same call as the reference extension.  thread_k / thread_n / sms choose
     CUDA tile shapes there and are accepted and ignored; max_par only sizes the
     reference's lock array, the same check is applied to `workspace`."""
-    if output_transpose:
-        raise RuntimeError("output_transpose=True is not supported (the reference's Python never passes it)")
     if workspace.numel() < size_n // 128 * max_par:
         raise RuntimeError(f"workspace must be of size at least {size_n // 128 * max_par}.")
-    return w4a16_gemm_ex(A, B, s, workspace, int(size_m), int(size_n), int(size_k))
+    return w4a16_gemm_ex(A, B, s, workspace, int(size_m), int(size_n), int(size_k),
+                         transpose_out=bool(output_transpose))
 
 
 def w4a16_dequant(B: torch.Tensor, s: torch.Tensor, size_n: int, size_k: int, want_codes: bool = False):
