@@ -247,6 +247,60 @@ def sweep(dev, gen, out_path):
         del weights
         torch.cuda.empty_cache()
 
+    # The linears and glue of one Llama-3.1-8B decoder layer around attention, per token batch:
+    # the reference's call sequence (q, k, v, rotary, o, gate, up, silu, multiply, down: 10
+    # launches, all on this build's kernels) against the fused one (qkv, rotary, o, gate/up with the
+    # SiLU epilogue, down: 5 launches).  Attention itself is left out of both.
+    from uniql_amd import layout
+    hid, nq, nkv, hd, inter = 4096, 32, 8, 128, 14336
+    for m in (1, 8):
+        copies = copies_for((hid * (nq + 2 * nkv) * hd + hid * hid + 3 * hid * inter) // 2)
+        sets = []
+        for _ in range(copies):
+            w = {name: make_weights(k_, n_, dev, gen) for name, k_, n_ in (
+                ("q", hid, nq * hd), ("k", hid, nkv * hd), ("v", hid, nkv * hd), ("o", nq * hd, hid),
+                ("gate", hid, inter), ("up", hid, inter), ("down", inter, hid))}
+            w["qkv"] = layout.concat_columns([w[n_][0] for n_ in "qkv"], [w[n_][1] for n_ in "qkv"])
+            w["gate_up"] = layout.interleave_gate_up(*w["gate"], *w["up"])
+            sets.append(w)
+        x = torch.randn((m, hid), device=dev, generator=gen).to(torch.float16)
+        attn = torch.randn((m, nq * hd), device=dev, generator=gen).to(torch.float16)
+        cos = torch.rand((1, m, hd), device=dev, generator=gen).to(torch.float16)
+        sin = torch.rand((1, m, hd), device=dev, generator=gen).to(torch.float16)
+        idx = torch.arange(hd, device=dev).to(torch.uint8).repeat(nkv, 1)
+        wsp = torch.zeros((2 * inter // 64) * 16, dtype=torch.int32, device=dev)
+
+        def lin(w, xin, n_, k_, **kw):
+            return ops.w4a16_linear(xin, w[0], w[1], wsp, n_, k_, **kw)
+
+        def unfused(i):
+            w = sets[i % copies]
+            q = lin(w["q"], x, nq * hd, hid)
+            k = lin(w["k"], x, nkv * hd, hid)
+            v = lin(w["v"], x, nkv * hd, hid)
+            ops.rope_indices_(q.view(1, m, nq, hd), k.view(1, m, nkv, hd), cos, sin, idx)
+            o = lin(w["o"], attn, hid, nq * hd)
+            h = torch.nn.functional.silu(lin(w["gate"], o, inter, hid)) * lin(w["up"], o, inter, hid)
+            return lin(w["down"], h, hid, inter), v
+
+        def fused(i):
+            w = sets[i % copies]
+            qkv = lin(w["qkv"], x, (nq + 2 * nkv) * hd, hid)
+            q, k = qkv[:, :nq * hd], qkv[:, nq * hd:(nq + nkv) * hd]
+            ops.rope_indices_(q.unflatten(1, (nq, hd)).unsqueeze(0), k.unflatten(1, (nkv, hd)).unsqueeze(0), cos, sin, idx)
+            o = lin(w["o"], attn, hid, nq * hd)
+            h = lin(w["gate_up"], o, 2 * inter, hid, silu_mul=True)
+            return lin(w["down"], h, hid, inter), qkv
+
+        sec_u, _ = time_graphs(unfused, copies, 200, 20)
+        sec_f, _ = time_graphs(fused, copies, 200, 20)
+        rows.append(dict(op="decoder_layer_linears_and_glue", m=m, us_fused=sec_f * 1e6, us_unfused=sec_u * 1e6,
+                         launches_fused=5, launches_unfused=10))
+        print("decoder layer (linears + rotary + MLP glue, no attention) M=%d: 5 launches %.2f us, 10 launches %.2f us"
+              % (m, sec_f * 1e6, sec_u * 1e6), file=sys.stderr, flush=True)
+        del sets
+        torch.cuda.empty_cache()
+
     # rotary embedding with gathered frequencies, Llama-3.1-8B heads (32 query, 8 key/value)
     for rows_x, d in ((1, 128), (1024, 128), (1024, 108), (4096, 128)):
         qs = [torch.randn((1, rows_x, 32, d), device=dev, generator=gen).to(torch.float16) for _ in range(4)]
