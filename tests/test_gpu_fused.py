@@ -236,13 +236,14 @@ def test_gate_up_module(gpu, in_f, width, bias):
         g16, u16 = gate(x).cpu().numpy(), up(x).cpu().numpy()
         want = O.mlp_gate_up(g16, u16)
         assert y.shape == (*shape[:-1], width)
-        # the gate/up sums may differ from the separate layers' in the last bit (other grid),
-        # which SiLU and the product carry through
+        # the gate/up sums may differ from the separate layers' in the last bit (other grid): one
+        # step of g is up to |u| steps of g in the product, plus the roundings of SiLU and of the
+        # product itself
         floor = 4e-2 if bias else 1e-4   # with a bias: one step of the un-biased products times |up|
-        assert_close16(y.cpu().numpy(), want, ulps=4, floor=floor, differing=5e-2)
+        assert_close16(y.cpu().numpy(), want, ulps=8, floor=floor, differing=5e-2)
         # and torch's own operators on the GPU give the same
         t = torch.nn.functional.silu(gate(x)) * up(x)
-        assert_close16(y.cpu().numpy(), t.cpu().numpy(), ulps=4, floor=floor, differing=5e-2)
+        assert_close16(y.cpu().numpy(), t.cpu().numpy(), ulps=8, floor=floor, differing=5e-2)
 
 
 def test_fused_call_errors(gpu):

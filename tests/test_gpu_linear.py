@@ -134,6 +134,24 @@ def test_tile_kernel_k_splits(gpu, splits):
     assert np.array_equal(y32, again)                          # integer accumulation: order-independent
 
 
+@pytest.mark.parametrize("mt", [1, 2])
+@pytest.mark.parametrize("m,k,n", [(32, 256, 128), (100, 1024, 256), (256, 4096, 512), (64, 768, 128), (33, 640, 256)])
+def test_tile_kernel_two_wave_quartets(gpu, m, k, n, mt):
+    """eight waves per workgroup, the quartets taking alternate K groups (an odd number of
+    groups, k = 640, falls back to one quartet)"""
+    p = make_linear_problem(m, k, n, seed=m + k)
+    ref = reference_product(p, exact=True)
+    flags = (1 << 2) | (mt << 16) | (2 << 20)
+    y32 = run_gemm(p, gpu, out_f32=True, flags=flags)
+    check_fp32_result(y32, p, ref, 1000)
+    y = run_gemm(p, gpu, flags=flags)
+    check_layer_output(y, ref)
+    # with K also split over workgroups (2 x 2 groups each at k = 1024)
+    if k % 512 == 0:
+        y32 = run_gemm(p, gpu, out_f32=True, flags=flags | (2 << 8))
+        check_fp32_result(y32, p, ref, 1000)
+
+
 def test_tile_kernel_per_column_and_stride(gpu):
     from uniql_amd import ops
     p = make_linear_problem(48, 384, 256, seed=21, per_column=True)

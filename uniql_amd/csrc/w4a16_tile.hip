@@ -118,31 +118,38 @@ __device__ __forceinline__ void store_eight_gated(const Epilogue& e, void* D, in
     }
 }
 
-template <int MT>
+template <int MT, int KW = 1>
 struct TileLds {
     static constexpr int kRows = 32 * MT;
     static constexpr int kXDwords = kRows * 64;        // X tile
     static constexpr int kBDwords = 4 * 2 * 256;       // 4 waves x 2 packed rows x 1 KiB
     static constexpr int kSDwords = 256;               // 4 copies of the strip's 256 bytes of scales
     static constexpr int kStageDwords = kXDwords + kBDwords + kSDwords;
-    static constexpr size_t kRingBytes = (size_t)kRing * kStageDwords * 4;
-    static constexpr size_t kRedBytes = (size_t)4 * 32 * 132 * 4;  // 4 waves x one 32-row M tile, fp32, padded rows
+    static constexpr size_t kRingBytes = (size_t)KW * kRing * kStageDwords * 4;  // one ring per wave quartet
+    static constexpr size_t kRedBytes = (size_t)KW * 4 * 32 * 132 * 4;  // every wave's 32-row M tile, fp32, padded rows
     static constexpr size_t kBytes = kRingBytes > kRedBytes ? kRingBytes : kRedBytes;
 };
 
 // EXT: the call uses something beyond the plain product (output cut or strided, bias, gated
 // pairs); the plain instantiation leaves that code out of the epilogue.
-template <int MT, bool EXT>
-__global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
-    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
-    using L = TileLds<MT>;
+// KW: quartets of waves per workgroup (1 or 2).  With two, the quartets take alternate K groups of
+// the same tile (each with its own LDS ring): two waves per SIMD cover each other's LDS and
+// expansion latencies, which is what small M tiles (little matrix work per group) lack when the
+// grid only gives a compute unit one workgroup.
+template <int MT, bool EXT, int KW>
+__global__ __launch_bounds__(256 * KW, 1) void w4a16_tile_kernel(const TileArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds_all[];
+    using L = TileLds<MT, KW>;
     constexpr int ROWS = L::kRows;
     constexpr int kXOps = ROWS / 16;        // X DMA instructions per wave and stage (4 rows each)
     constexpr int kStageOps = kXOps + 3;    // + two packed rows + scales
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int w8 = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int w = w8 & 3;      // role inside the quartet: packed rows w and w + 4 of a group
+    const int par = w8 >> 2;   // quartet: takes K groups par, par + KW, ... of the workgroup's range
+    uint32_t* lds = lds_all + par * (kRing * L::kStageDwords);  // this quartet's ring
     // MFMA view of the lane
     const int s = lane & 31;
     const int h = lane >> 5;
@@ -163,9 +170,10 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     const int m0 = mblock * ROWS;
 
     const int N4 = a.N >> 1;
-    const int g_begin = split * a.gps;
-    const int g_end = (g_begin + a.gps < a.G) ? (g_begin + a.gps) : a.G;
-    const int ngroups = g_end - g_begin;
+    const int g_first = split * a.gps;
+    const int g_end = (g_first + a.gps < a.G) ? (g_first + a.gps) : a.G;
+    const int g_begin = g_first + par;
+    const int ngroups = (g_end - g_first) / KW;  // per quartet; the plan makes the range a multiple of KW
 
     // packed rows w and w + 4 of every group; DMA lane (c8', ch', kq') fetches piece 32 ch' + 4 c8' + kq'
     const uint32_t piece_off = (uint32_t)((dslot >> 3) * 32 + 4 * (dslot & 7) + dkq);
@@ -366,9 +374,9 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     h8 bw;
     if (ngroups > 0) {
         issue_stage(g_begin, 0);
-        issue_stage(ngroups > 1 ? g_begin + 1 : g_last, 1);
+        issue_stage(ngroups > 1 ? g_begin + KW : g_last, 1);
 #pragma unroll
-        for (int idx = 0; idx < kDmaA; ++idx) issue_piece(group_or_last(g_begin + 2), 2, idx);
+        for (int idx = 0; idx < kDmaA; ++idx) issue_piece(group_or_last(g_begin + 2 * KW), 2, idx);
         UNIQL_WAIT_VMCNT(kStageOps + kDmaA);
         __builtin_amdgcn_s_barrier();
         read_words(0, 0);
@@ -379,12 +387,12 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     for (int it = 0; it < ngroups; ++it) {
         const int slot_next = slot + 1 == kRing ? 0 : slot + 1;
         const int slot_prev = slot == 0 ? kRing - 1 : slot - 1;   // holds stage it+2
-        half_stage(0, xa0, bw, kDmaA, kDmaB, group_or_last(g_begin + it + 2), slot_prev, [&](int i) __attribute__((always_inline)) {
+        half_stage(0, xa0, bw, kDmaA, kDmaB, group_or_last(g_begin + KW * (it + 2)), slot_prev, [&](int i) __attribute__((always_inline)) {
             if (i < MT) read_xa_one(xa1, slot, 1, i);
         });
         UNIQL_WAIT_VMCNT(kStageOps);   // stage it+1 has landed; only stage it+2's loads are outstanding
         __builtin_amdgcn_s_barrier();
-        half_stage(1, xa1, bw, 0, kDmaA, group_or_last(g_begin + it + 3), slot, [&](int i) __attribute__((always_inline)) {
+        half_stage(1, xa1, bw, 0, kDmaA, group_or_last(g_begin + KW * (it + 3)), slot, [&](int i) __attribute__((always_inline)) {
             if (i == 0) read_words(1, slot_next);
             if (i >= 1 && i <= MT) read_xa_one(xa0, slot_next, 0, i - 1);
         });
@@ -408,7 +416,8 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
     // partials of two (row, 8 consecutive columns) units and stores each unit with one 16-byte
     // store.
     constexpr int kRedStride = 132;
-    float* red = reinterpret_cast<float*>(lds);  // [4 waves][32 rows][132]
+    float* red = reinterpret_cast<float*>(lds_all);  // [4 KW waves][32 rows][132]
+    constexpr int NW = 4 * KW;
     const bool split_k = a.splits > 1;
     const bool gated = EXT && a.epi.gated != 0;  // uniform
 #pragma unroll
@@ -416,7 +425,7 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
         if (m0 + mt * 32 < a.M) {  // uniform
             if (mt > 0) __syncthreads();
             {
-                float* wred = red + w * 32 * kRedStride + s * kRedStride + 4 * h;
+                float* wred = red + w8 * 32 * kRedStride + s * kRedStride + 4 * h;
 #pragma unroll
                 for (int op = 0; op < 4; ++op)
 #pragma unroll
@@ -428,16 +437,15 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
             if (!split_k) {
                 // gated: the 32 x 64 output block is 256 units, one per thread (columns c0 and
                 // c0 + 64 of the strip); else 512 units, two per thread
-                const int units = gated ? 1 : 2;
-                for (int u2 = 0; u2 < units; ++u2) {
-                    const int unit = tid + 256 * u2;
+                const int units = gated ? 256 : 512;
+                for (int unit = tid; unit < units; unit += 256 * KW) {
                     const int row = gated ? unit >> 3 : unit >> 4;
                     const int c0 = gated ? (unit & 7) * 8 : (unit & 15) * 8;
                     const int m = m0 + mt * 32 + row;
                     const float* src = red + row * kRedStride + c0;
                     f4 lo = *reinterpret_cast<const f4*>(src), hi = *reinterpret_cast<const f4*>(src + 4);
 #pragma unroll
-                    for (int ww = 1; ww < 4; ++ww) {
+                    for (int ww = 1; ww < NW; ++ww) {
                         lo += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride);
                         hi += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride + 4);
                     }
@@ -462,7 +470,7 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
                     } else {
                         f4 ulo = *reinterpret_cast<const f4*>(src + 64), uhi = *reinterpret_cast<const f4*>(src + 68);
 #pragma unroll
-                        for (int ww = 1; ww < 4; ++ww) {
+                        for (int ww = 1; ww < NW; ++ww) {
                             ulo += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride + 64);
                             uhi += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride + 68);
                         }
@@ -473,12 +481,14 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
                 // K is also split over workgroups: one atomic per element, neighbouring lanes on
                 // neighbouring words (a wave touches 512 contiguous bytes per instruction)
                 const int col_out = tid & 127;
-                for (int i = 0; i < 16; ++i) {
-                    const int row = (tid >> 7) + 2 * i;
+                for (int i = 0; i < 16 / KW; ++i) {
+                    const int row = (tid >> 7) + 2 * KW * i;
                     const int m = m0 + mt * 32 + row;
                     if (m >= a.M) continue;
                     const float* src = red + row * kRedStride + col_out;
-                    const float sum = (src[0] + src[32 * kRedStride]) + (src[64 * kRedStride] + src[96 * kRedStride]);
+                    float sum = (src[0] + src[32 * kRedStride]) + (src[64 * kRedStride] + src[96 * kRedStride]);
+                    if (KW == 2)
+                        sum += (src[128 * kRedStride] + src[160 * kRedStride]) + (src[192 * kRedStride] + src[224 * kRedStride]);
                     const int n_out = 128 * strip + col_out;
                     unsigned long long* word = a.accum + (size_t)m * a.N + n_out;
                     if (!gated) {
@@ -495,8 +505,10 @@ __global__ __launch_bounds__(256, 1) void w4a16_tile_kernel(const TileArgs a) {
                         }
                     } else if (col_out < 64) {
                         const float* usrc = src + 64;
-                        const float usum =
-                            (usrc[0] + usrc[32 * kRedStride]) + (usrc[64 * kRedStride] + usrc[96 * kRedStride]);
+                        float usum = (usrc[0] + usrc[32 * kRedStride]) + (usrc[64 * kRedStride] + usrc[96 * kRedStride]);
+                        if (KW == 2)
+                            usum += (usrc[128 * kRedStride] + usrc[160 * kRedStride]) +
+                                    (usrc[192 * kRedStride] + usrc[224 * kRedStride]);
                         float total_g, total_u;
                         if (accum_add_pair(word, word + 64, sum, usum, a.splits, total_g, total_u)) {
                             finish_store_gated(a.epi, a.D, m, 64 * strip + col_out, total_g, total_u);
@@ -514,8 +526,9 @@ static inline int ceil_div_i(int a, int b) { return (a + b - 1) / b; }
 
 struct TilePlan {
     int mtiles, splits, gps;
+    int quartets;  // wave quartets per workgroup (1 or 2)
 };
-static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_override = 0);
+static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_override = 0, int kw_override = 0);
 
 size_t tile_accum_bytes(int m, int n, int k) {
     // one word per output element, only when the plan splits K over workgroups
@@ -529,19 +542,25 @@ size_t tile_accum_bytes(int m, int n, int k) {
 //     is expanded twice per 128 rows), a last round of at most 256 costs 0.85;
 //   * MT = 1: up to four share a compute unit: 0.62 for at most 256 workgroups, 0.88 for at most
 //     512, 1.62 per started round of 1024;
+//   * a grid that gives a compute unit at most one MT = 1 or MT = 2 workgroup runs faster with two
+//     wave quartets per workgroup (factors 0.85 and 0.92);
 //   * the exchange of partial sums costs one 64-bit atomic per output element and K split,
 //     about 150 G atomics/s for the chip.
 // So: the MT with the cheapest grid; K splits only for MT = 1 grids that cannot fill the chip,
-// and only while the atomics cost less than the K loop they save.
-static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_override) {
+// and only while the atomics cost less than the K loop they save; two quartets whenever the final
+// grid has at most 256 workgroups of MT <= 2 and every workgroup gets an even number of groups.
+static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_override, int kw_override) {
     TilePlan p;
     const int strips = n / 128, G = k / 128;
+    const bool even_g = G % 2 == 0;
     const int64_t t4 = (int64_t)strips * ceil_div_i(m, 128), t2 = (int64_t)strips * ceil_div_i(m, 64);
     const int64_t t1 = (int64_t)strips * ceil_div_i(m, 32);
     const double cost4 = (double)((t4 + 255) / 256);
     const int64_t rem2 = t2 % 512;
-    const double cost2 = 1.08 * (double)(t2 / 512) + (rem2 == 0 ? 0.0 : (rem2 <= 256 ? 0.85 : 1.08));
-    const double cost1 = t1 <= 256 ? 0.62 : (t1 <= 512 ? 0.88 : 1.62 * (double)((t1 + 1023) / 1024));
+    double cost2 = 1.08 * (double)(t2 / 512) + (rem2 == 0 ? 0.0 : (rem2 <= 256 ? 0.85 : 1.08));
+    double cost1 = t1 <= 256 ? 0.62 : (t1 <= 512 ? 0.88 : 1.62 * (double)((t1 + 1023) / 1024));
+    if (even_g && t2 <= 256) cost2 *= 0.92;
+    if (even_g && t1 <= 256) cost1 *= 0.85;
     p.mtiles = 4;
     if (cost2 < cost4 && cost2 <= cost1) p.mtiles = 2;
     else if (cost1 < cost4) p.mtiles = 1;
@@ -566,27 +585,43 @@ static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_overr
     if (splits > 255) splits = 255;
     p.gps = ceil_div_i(G, splits);
     p.splits = ceil_div_i(G, p.gps);
+    // two quartets take alternate groups: every workgroup's range must hold an even number
+    p.quartets = 1;
+    const bool want2 = kw_override == 2 || (kw_override == 0 && tiles * p.splits <= 256);
+    if (want2 && p.mtiles <= 2 && even_g) {
+        const int gps2 = p.gps + (p.gps & 1);
+        if (splits_override == 0 || gps2 == p.gps) {
+            p.gps = gps2;
+            p.splits = ceil_div_i(G, p.gps);
+            p.quartets = 2;
+        }
+    }
     return p;
 }
 
-template <int MT, bool EXT>
+template <int MT, bool EXT, int KW>
 static hipError_t tile_launch_one(const TileArgs& a, int grid, hipStream_t stream) {
-    const size_t shmem = TileLds<MT>::kBytes;
-    auto kern = &w4a16_tile_kernel<MT, EXT>;
+    const size_t shmem = TileLds<MT, KW>::kBytes;
+    auto kern = &w4a16_tile_kernel<MT, EXT, KW>;
     if (shmem > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return e;
     }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), shmem, stream, a);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256 * KW), shmem, stream, a);
     return hipGetLastError();
 }
 
+template <int MT, int KW>
+static hipError_t tile_launch_ext(const TileArgs& a, bool ext, int grid, hipStream_t stream) {
+    return ext ? tile_launch_one<MT, true, KW>(a, grid, stream) : tile_launch_one<MT, false, KW>(a, grid, stream);
+}
+
 // tune: bits 0..7 force the number of K splits, bits 8..11 the number of 32-row M tiles per
-// workgroup (0 = choose)
+// workgroup, bits 12..13 the number of wave quartets (0 = choose)
 int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, const Epilogue& epi, void* accum,
                 size_t accum_bytes, int m, int n, int k, int groups, unsigned tune, hipStream_t stream) {
-    const TilePlan plan = tile_plan(m, n, k, (int)(tune & 0xffu), (int)((tune >> 8) & 0xfu));
+    const TilePlan plan = tile_plan(m, n, k, (int)(tune & 0xffu), (int)((tune >> 8) & 0xfu), (int)((tune >> 12) & 0x3u));
     if (plan.splits > 1 && (!accum || accum_bytes < (size_t)m * n * sizeof(unsigned long long)))
         return UNIQL_E_WORKSPACE;
     TileArgs a;
@@ -610,11 +645,11 @@ int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* 
     hipError_t e;
     const bool ext = epi.gated || epi.bias || epi.transpose || epi.n_store != n || epi.ldd != n || !epi.vec_ok;
     if (plan.mtiles == 1)
-        e = ext ? tile_launch_one<1, true>(a, (int)grid, stream) : tile_launch_one<1, false>(a, (int)grid, stream);
+        e = plan.quartets == 2 ? tile_launch_ext<1, 2>(a, ext, (int)grid, stream) : tile_launch_ext<1, 1>(a, ext, (int)grid, stream);
     else if (plan.mtiles == 2)
-        e = ext ? tile_launch_one<2, true>(a, (int)grid, stream) : tile_launch_one<2, false>(a, (int)grid, stream);
+        e = plan.quartets == 2 ? tile_launch_ext<2, 2>(a, ext, (int)grid, stream) : tile_launch_ext<2, 1>(a, ext, (int)grid, stream);
     else
-        e = ext ? tile_launch_one<4, true>(a, (int)grid, stream) : tile_launch_one<4, false>(a, (int)grid, stream);
+        e = tile_launch_ext<4, 1>(a, ext, (int)grid, stream);
     return e == hipSuccess ? UNIQL_OK : UNIQL_E_LAUNCH;
 }
 
