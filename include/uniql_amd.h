@@ -45,7 +45,7 @@ enum {
     /* tuning hooks, 0 = choose.  Streaming kernel: bits 8..15 K-groups per wavefront,
        bits 16..20 wavefronts per workgroup (4 or 8).
        Tiled kernel: bits 8..15 number of K splits over workgroups, bits 16..19 row tiles of 32
-       per workgroup (1, 2 or 4). */
+       per workgroup (1, 2 or 4), bits 20..21 wave quartets per workgroup (1 or 2). */
 };
 
 int uniql_abi_version(void);
