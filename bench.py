@@ -42,7 +42,7 @@ LLC_BYTES = 256 << 20
 # HBM bytes per launch of the default workload (mean over the four linears) from two
 # rocprofv3 --pmc runs of this file, FETCH_SIZE and WRITE_SIZE, each scaled by the reading for a
 # 128 MiB elementwise copy (--pmc-calibrate): factors 2.000 and 1.000.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28734222
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28727290
 
 LLAMA_DECODE = [("qkv", 4096, 6144), ("o_proj", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
 PRUNED = [("q_pruned", 4096, 3584, 0), ("o_pruned", 3456, 4096, 0), ("gate_up_pruned", 4096, 24320, 0),
@@ -87,11 +87,14 @@ class Layer:
         return ops.w4a16o16_gemm(self.x, b, s, self.ws, self.m, self.n, self.k, False, -1, -1, -1, 16)
 
 
+GRAPH_STEPS = 40   # steps captured per HIP graph (a decode step of a 32-layer model replays more kernels than that)
+
+
 def time_graphs(run_step, n_variants, steps, warmup):
     """Times exactly `steps` calls of run_step(i), i cycling over n_variants, as HIP graph
-    replays: one graph holds n_variants consecutive steps (a second, shorter one the
-    remainder), so the per-replay launch cost is shared by many kernels.  Returns
-    (seconds per step from events on the launch stream, wall seconds per step)."""
+    replays: one graph holds a multiple of n_variants consecutive steps (about GRAPH_STEPS; a
+    second, shorter graph the remainder), so the per-replay launch cost is shared by many
+    kernels.  Returns (seconds per step from events on the launch stream, wall seconds per step)."""
     import torch
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -109,15 +112,16 @@ def time_graphs(run_step, n_variants, steps, warmup):
                 keep.append(run_step(i))
         return g
 
-    full = capture(n_variants)
-    rest = capture(steps % n_variants) if steps % n_variants else None
-    for _ in range(max(1, warmup // n_variants)):
+    per_graph = n_variants * max(1, min(steps, GRAPH_STEPS) // n_variants)
+    full = capture(per_graph)
+    rest = capture(steps % per_graph) if steps % per_graph else None
+    for _ in range(max(1, warmup // per_graph)):
         full.replay()
     torch.cuda.synchronize()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     t0 = time.perf_counter()
     start.record()
-    for _ in range(steps // n_variants):
+    for _ in range(steps // per_graph):
         full.replay()
     if rest is not None:
         rest.replay()
