@@ -268,11 +268,30 @@ def test_side_stream_and_graph_replay(gpu):
     dev_in = [to_gpu(p, gpu) for p in problems]
     ws = [workspace_for(p["n"], gpu) for p in problems]
 
+    bias = torch.linspace(-1, 1, 200, device=gpu).half()
+    pair_bias = torch.linspace(-1, 1, 512, device=gpu).half()
+    q0 = torch.randn(1, 70, 4, 16, generator=torch.Generator().manual_seed(5)).half().to(gpu)
+    k0 = torch.randn(1, 70, 2, 16, generator=torch.Generator().manual_seed(6)).half().to(gpu)
+    cos = torch.rand(1, 70, 16, generator=torch.Generator().manual_seed(7)).half().to(gpu)
+    idx = torch.arange(16, dtype=torch.uint8, device=gpu).repeat(2, 1)
+    table = (torch.randn(64, 128, generator=torch.Generator().manual_seed(8)) * 0.1).half().to(gpu)
+
     def run_all():
         outs = []
         for i, (p, (x, b, s)) in enumerate(zip(problems, dev_in)):
             kw = dict(had_block=128, had_scale=128 ** -0.5) if i == 2 else {}
             outs.append(ops.w4a16_gemm_ex(x, b, s, ws[i], p["m"], p["n"], p["k"], **kw))
+        # the layer call with its epilogues: cut + bias (tiled kernel), gated pairs with K split over
+        # workgroups (streaming kernel: the pair exchange through the accumulator words)
+        x, b, s = dev_in[1]
+        outs.append(ops.w4a16_linear(x[:, :1400], b, s, ws[1], 256, 1408, out_features=200, bias=bias))
+        x, b, s = dev_in[0]
+        outs.append(ops.w4a16_linear(x, b, s, ws[0], 512, 4096, silu_mul=True, bias=pair_bias))
+        # rotary embedding (in place: work on copies), embedding-table quantiser
+        q, k = q0.clone(), k0.clone()
+        ops.rope_indices_(q, k, cos, cos, idx)
+        outs += [q, k]
+        outs += list(ops.w4_embedding_quantize(table))
         return outs
 
     eager = [y.clone() for y in run_all()]
@@ -289,7 +308,7 @@ def test_side_stream_and_graph_replay(gpu):
         captured = run_all()
     for rep in range(3):
         for y in captured:
-            y.fill_(float("nan"))
+            y.fill_(float("nan")) if y.is_floating_point() else y.fill_(-1)
         graph.replay()
         torch.cuda.synchronize()
         for a, b in zip(eager, captured):
