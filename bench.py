@@ -1,6 +1,6 @@
 """Benchmark of the W4A16 hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--sweep [--sweep-json PATH]] [--no-cpu]
 
 Default workload (the line the driver records): the decode sweep's M = 1 column,
 "llama31_8b_decode_layer_m1": one step = the four W4A16 GEMVs of a Llama-3.1-8B
@@ -9,18 +9,19 @@ decoder layer at M = 1 (fused qkv 4096->6144, o_proj 4096->4096, fused gate_up
 Inputs are synthetic (codes U{0..15}, scales U[0.004,0.02], x ~ N(0,1), seed 1234) and
 resident in HBM before the timed region.  Successive steps use different weight
 copies whose total size exceeds the 256 MB last-level cache, so the weights come
-from HBM, not from cache.  Steps are replayed as HIP graphs (one per weight copy)
-so that launch overhead is the GPU's, not Python's.
+from HBM, not from cache.  Steps are replayed as HIP graphs of about 40 steps each, so
+that launch overhead is the GPU's, not Python's, and replay boundaries are rare.
 
 value = algorithmic bytes per step / time per step  (GB/s), algorithmic bytes of a
 linear = K N / 2 + (K/128) N 2 + M K 2 + M N 2.  The same JSON line carries, under
 "prefill_gemm_m1024", the other half of the metric: the four linears at M = 1024 through
 the tiled MFMA kernel (TFLOP/s = 2 M K N / time, against 2.5 PFLOP/s dense fp16).
 
---sweep additionally prints (stderr) and writes (gpurun_out/bench_sweep.json) the
-per-shape tables: decode M in {1,2,4,8}, prefill M in {256,1024,4096}, the pruned
-Llama shapes with the fused 128-block rotation, the Mamba2 shapes, the embedding
-gather and the standalone transform.
+--sweep additionally prints (stderr) and writes (--sweep-json, default bench_sweep.json in the
+working directory) the per-shape tables: decode M in {1,2,4,8}, prefill M in {256,1024,4096},
+the pruned Llama shapes with the fused 128-block rotation, the Mamba2 shapes, the embedding
+gather, the standalone transform, the MLP front with the SiLU epilogue against the unfused
+sequence, a decoder layer's linears and glue as 5 against 10 launches, and the rotary kernel.
 """
 from __future__ import annotations
 
@@ -319,7 +320,8 @@ def sweep(dev, gen, out_path):
         print("rope rows=%d head_dim=%d: %.2f us %.1f GB/s" % (rows_x, d, sec * 1e6, per / sec / 1e9),
               file=sys.stderr, flush=True)
 
-    os.makedirs(os.path.dirname(out_path), exist_ok=True)
+    if os.path.dirname(out_path):
+        os.makedirs(os.path.dirname(out_path), exist_ok=True)
     with open(out_path, "w") as f:
         json.dump(rows, f, indent=1)
 
@@ -331,6 +333,7 @@ def main():
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=40)
     ap.add_argument("--sweep", action="store_true")
+    ap.add_argument("--sweep-json", default="bench_sweep.json", help="where --sweep writes its table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--pmc-calibrate", action="store_true",
                     help="also launch three plain elementwise copies of 128 MiB (read 128 MiB, write 128 MiB each) "
@@ -405,7 +408,7 @@ def main():
                      "unit": "TFLOP/s", "frac": round(tot_flops / tot_sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                      "kernel": "w4a16_tile_kernel<MT> (MT = 4, or 2 for the 6144-wide qkv)"}}
     if args.sweep:
-        sweep(dev, gen, os.path.join(ROOT, "gpurun_out", "bench_sweep.json"))
+        sweep(dev, gen, args.sweep_json)
     if not args.no_cpu:
         result["cpu_baseline"] = cpu_baseline()
     print(json.dumps(result), flush=True)
