@@ -110,7 +110,7 @@ def time_graphs(run_step, n_variants, steps, warmup):
         g = torch.cuda.CUDAGraph()
         with torch.cuda.graph(g):
             for i in range(count):
-                keep.append(run_step(i))
+                keep.append(run_step(i % n_variants))
         return g
 
     per_graph = n_variants * max(1, min(steps, GRAPH_STEPS) // n_variants)

@@ -193,14 +193,120 @@ __global__ __launch_bounds__(1024) void fwht_f16_kernel(const u32x4* __restrict_
     }
 }
 
+// Long rows (L >= 4096), fp16: two LDS exchanges instead of one per four index bits.
+//   load    every thread takes L/8/T sixteen-byte chunks (consecutive lanes on consecutive chunks),
+//           transforms index bits 0..2 in registers and writes fp32 to LDS;
+//   middle  index bits 3 .. n-6 in passes of up to five bits (32 values per task in registers);
+//   final   the top five bits: a thread reads two neighbouring values at 32 strides of L/32,
+//           transforms, scales, rounds and stores 4 bytes per stride: consecutive lanes store
+//           consecutive words, no trip back through LDS.
+// The stages run in ascending bit order like everywhere else, so the fp32 sums are associated
+// the same way and the result is the same bit for bit.  T = L / 64 threads per row.
+__global__ __launch_bounds__(512) void fwht_f16_wide_kernel(const u32x4* __restrict__ x, uint32_t* __restrict__ y,
+                                                           int L, int log2L, float scale) {
+    extern __shared__ __attribute__((aligned(16))) float fbuf[];
+    const int tid = threadIdx.x, nthreads = blockDim.x;
+    const int chunks = L >> 3;
+    const u32x4* xp = x + (size_t)blockIdx.x * chunks;
+    uint32_t* yp = y + (size_t)blockIdx.x * (L >> 1);
+    constexpr int kChunksPerThread = 8;  // chunks / nthreads = (L / 8) / (L / 64)
+    u32x4 v[kChunksPerThread];
+#pragma unroll
+    for (int i = 0; i < kChunksPerThread; ++i) v[i] = xp[tid + i * nthreads];
+#pragma unroll
+    for (int i = 0; i < kChunksPerThread; ++i) {
+        float f[8];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const h2 hv = bits_to_h2(v[i][p]);
+            f[2 * p] = (float)hv.x;
+            f[2 * p + 1] = (float)hv.y;
+        }
+#pragma unroll
+        for (int h = 1; h < 8; h <<= 1) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                if ((e & h) == 0) {
+                    const float p = f[e], q = f[e + h];
+                    f[e] = p + q;
+                    f[e + h] = p - q;
+                }
+            }
+        }
+        float* dst = fbuf + fwht_pad(8 * (tid + i * nthreads));
+        *reinterpret_cast<f4*>(dst) = f4{f[0], f[1], f[2], f[3]};
+        *reinterpret_cast<f4*>(dst + 4) = f4{f[4], f[5], f[6], f[7]};
+    }
+    __syncthreads();
+    int lo = 3;
+    const int top = log2L - 5;  // first bit of the final phase
+    while (lo < top) {
+        const int left = top - lo;
+        if (left >= 5) {
+            fwht_pass_padded<5>(fbuf, L, lo, tid, nthreads);
+            lo += 5;
+        } else if (left == 4) {
+            fwht_pass_padded<4>(fbuf, L, lo, tid, nthreads);
+            lo += 4;
+        } else if (left == 3) {
+            fwht_pass_padded<3>(fbuf, L, lo, tid, nthreads);
+            lo += 3;
+        } else if (left == 2) {
+            fwht_pass_padded<2>(fbuf, L, lo, tid, nthreads);
+            lo += 2;
+        } else {
+            fwht_pass_padded<1>(fbuf, L, lo, tid, nthreads);
+            lo += 1;
+        }
+        __syncthreads();
+    }
+    // final phase: values 2 tid, 2 tid + 1 at the 32 strides of L / 32
+    const int stride = L >> 5;
+    float a[32], b[32];
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+        const float* src = fbuf + fwht_pad(2 * tid + j * stride);
+        a[j] = src[0];
+        b[j] = src[1];
+    }
+#pragma unroll
+    for (int h = 1; h < 32; h <<= 1) {
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            if ((j & h) == 0) {
+                const float p = a[j], q = a[j + h];
+                a[j] = p + q;
+                a[j + h] = p - q;
+                const float r = b[j], t = b[j + h];
+                b[j] = r + t;
+                b[j + h] = r - t;
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 32; ++j) {
+        h2 r;
+        r.x = scaled_to_half(a[j], scale);
+        r.y = scaled_to_half(b[j], scale);
+        yp[tid + j * (stride >> 1)] = h2_to_bits(r);
+    }
+}
+
 static int fwht_f16_launch(const void* x, void* y, int64_t pieces, int block, float scale, hipStream_t stream) {
     int log2L = 0;
     while ((1 << log2L) < block) ++log2L;
     const size_t shmem = (size_t)(block + (block >> 7) * 8) * sizeof(float);
     if (shmem > 64 * 1024) {
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(&fwht_f16_kernel),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess ||
+            hipFuncSetAttribute(reinterpret_cast<const void*>(&fwht_f16_wide_kernel),
                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem) != hipSuccess)
             return UNIQL_E_LAUNCH;
+    }
+    if (block >= 4096) {
+        hipLaunchKernelGGL(fwht_f16_wide_kernel, dim3((unsigned)pieces), dim3(block / 64), shmem, stream,
+                           reinterpret_cast<const u32x4*>(x), reinterpret_cast<uint32_t*>(y), block, log2L, scale);
+        return UNIQL_OK;
     }
     const int threads = block / 8 < 1024 ? block / 8 : 1024;
     hipLaunchKernelGGL(fwht_f16_kernel, dim3((unsigned)pieces), dim3(threads), shmem, stream,
