@@ -180,7 +180,7 @@ def sweep(dev, gen, out_path):
         per = linear_bytes(m, k, n)
         copies = copies_for(k * n // 2) if m <= 64 else 2
         layer = Layer(name, k, n, m, copies, dev, gen, had_block)
-        sec, _ = time_graphs(lambda i: layer.run(i), copies, steps, 20)
+        sec, _ = time_graphs(lambda i: layer.run(i), copies, steps, max(20, steps // 2))
         row = dict(op=name, m=m, k=k, n=n, had_block=had_block, us=sec * 1e6, gbs=per / sec / 1e9,
                    hbm_frac=per / sec / 1e9 / HBM_PEAK_GBS, tflops=linear_flops(m, k, n) / sec / 1e12,
                    mfma_frac=linear_flops(m, k, n) / sec / 1e12 / MFMA_F16_PEAK_TFLOPS)
@@ -196,10 +196,10 @@ def sweep(dev, gen, out_path):
             bench_linear(name, k, n, m)
     for m in (256, 1024, 4096):
         for name, k, n in LLAMA_DECODE:
-            bench_linear(name, k, n, m, steps=20)
+            bench_linear(name, k, n, m, steps=100)
     for m in (1, 1024):
         for name, k, n, hb in PRUNED + MAMBA:
-            bench_linear(name, k, (n + 255) // 256 * 256, m, hb, steps=200 if m == 1 else 20)
+            bench_linear(name, k, (n + 255) // 256 * 256, m, hb, steps=200 if m == 1 else 100)
 
     # embedding gather: V = 256000, D = 4096, 2048 ids
     v, d, t = 256000, 4096, 2048
@@ -240,7 +240,7 @@ def sweep(dev, gen, out_path):
             y = ops.w4a16_linear(x, b, sc, ws, 2 * width, k).view(m, width // 64, 2, 64)
             return torch.nn.functional.silu(y[:, :, 0]) * y[:, :, 1]
 
-        steps = 200 if m <= 64 else 20
+        steps = 200 if m <= 64 else 100
         sec_f, _ = time_graphs(fused, copies, steps, 20)
         sec_u, _ = time_graphs(unfused, copies, steps, 20)
         per = linear_bytes(m, k, 2 * width) - m * width * 2   # half the output bytes
@@ -394,7 +394,8 @@ def main():
     per_shape, tot_flops, tot_sec = {}, 0.0, 0.0
     for name, k, n in LLAMA_DECODE:
         layer = Layer(name, k, n, pm, 2, dev, gen)
-        sec, _ = time_graphs(lambda i: layer.run(i), 2, 20, 4)
+        # the clocks of a chip that was idle take a few milliseconds to settle: 40 untimed steps first
+        sec, _ = time_graphs(lambda i: layer.run(i), 2, 100, 40)
         fl = linear_flops(pm, k, n)
         per_shape[name] = {"us": round(sec * 1e6, 2), "tflops": round(fl / sec / 1e12, 1)}
         tot_flops += fl
