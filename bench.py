@@ -383,7 +383,7 @@ def main():
                    "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "wall_ms_per_step": round(wall_per_step * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "w4a16_stream_kernel<MT=1,HAD=false> (all four launches of a step)", "launches_per_step": launches,
+                     "kernel": "w4a16_stream_kernel<RC=1,HAD=false> (all four launches of a step)", "launches_per_step": launches,
                      "avg_launch_us": round(kernel_us, 3), "bytes_per_launch": step_bytes // launches},
     }
     del layers

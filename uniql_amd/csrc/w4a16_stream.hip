@@ -57,13 +57,15 @@ struct StreamArgs {
     int per_column;       // 1: a single scale row (per-column scales)
     int upw;              // groups per wave
     int splits;           // workgroups along K per strip
-    int xrows;            // activation rows staged per wave: multiple of 4, >= min(M, 16 MT)
+    int xrows;            // activation rows staged per wave: M rounded up to a multiple of 4
     int k_valid;          // columns of X that exist (multiple of 8); the rest of K counts as zeros
     float had_scale;
     Epilogue epi;
 };
 
-// MT: 16-row tiles of M per workgroup.  RC: row class, an upper bound of M for MT = 1
+// One launch covers up to 16 rows of X (the rows of one MFMA tile); more rows run as further
+// launches over the same weights, which only the forcing flag asks for: from 17 rows on the
+// tiled kernel is faster.  RC: row class, an upper bound of M
 // (1, 2, 4, 8, 16): it fixes NV, how many of the four output rows of a lane's accumulator
 // quad are real, and XQ, how many quads of activation rows are loaded and staged.  WAVES:
 // wavefronts per workgroup (4 or 8); with 8 a workgroup can cover all of K for shapes with
@@ -73,12 +75,12 @@ struct StreamArgs {
 // uses something beyond the plain product (input shorter than K, output cut or strided, bias,
 // gated pairs); the plain instantiation leaves all of that code out, which at a few
 // microseconds per launch is measurable (instruction fetch).
-template <int MT, int RC, bool HAD, int WAVES, bool EXT>
-__global__ __launch_bounds__(64 * WAVES, (MT == 1 ? 3 : (MT == 2 ? 2 : 1)))
+template <int RC, bool HAD, int WAVES, bool EXT>
+__global__ __launch_bounds__(64 * WAVES, 3)
 void w4a16_stream_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     constexpr int NV = RC < 4 ? RC : 4;
-    constexpr int XQ = MT > 1 ? 4 : (RC + 3) / 4;
+    constexpr int XQ = (RC + 3) / 4;
     constexpr int RPW = 4;  // row pairs (32 K values each) per group
 
     const int tid = threadIdx.x;
@@ -102,27 +104,20 @@ void w4a16_stream_kernel(const StreamArgs a) {
     const u32x4* strip_w = a.B + (size_t)strip * 64;
     const half_t* strip_s = a.S + (size_t)strip * 128;
 
-    float acc[MT][8][NV];
+    float acc[8][NV];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt)
+    for (int jb = 0; jb < 8; ++jb)
 #pragma unroll
-        for (int jb = 0; jb < 8; ++jb)
-#pragma unroll
-            for (int v = 0; v < NV; ++v) acc[mt][jb][v] = 0.f;
+        for (int v = 0; v < NV; ++v) acc[jb][v] = 0.f;
 
     uint32_t* xs = lds + (size_t)w * a.xrows * kXsStride;  // this wave's staging rows
     // Staged row layout (dwords): the pair of K values 2d, 2d+1 of the group, d = 16 rp + kq' + 4 t,
     // sits at dword 16 rp + 4 kq' + t, so that the A operand of lane (row, kq') for row pair rp
     // is one 16-byte read; pairs with odd t (K rows 8..15 of a packed row) are stored divided
     // by 16.  Dword 64 of the row holds 8 * 2^-24 * (sum of the row's values) as fp32.
-    // MFMA row `slot` of tile mt reads staged row min(16 mt + slot, xrows - 1): rows past M
-    // only feed output rows that are never stored.
-    int xrow_of[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) {
-        const int r = mt * 16 + slot;
-        xrow_of[mt] = (r < a.xrows ? r : a.xrows - 1) * kXsStride + 4 * kq;
-    }
+    // MFMA row `slot` reads staged row min(slot, xrows - 1): rows past M only feed output rows
+    // that are never stored.
+    const int xrow_of = (slot < a.xrows ? slot : a.xrows - 1) * kXsStride + 4 * kq;
     // where this lane's staged quad goes: lane `slot` holds pairs d = 4 slot + i
     const int stage_off = 16 * (slot >> 2) + (slot & 3);
     const half_t stage_mul = (slot & 1) ? (half_t)0.0625f : (half_t)1.0f;
@@ -132,19 +127,16 @@ void w4a16_stream_kernel(const StreamArgs a) {
 
     u32x4 wq[2 * RPW];
     u32x4 sc;
-    u32x4 xv[MT][XQ];
+    u32x4 xv[XQ];
     // everything group g needs from memory: activations first (small, they gate the LDS
     // staging), then scales, then the eight packed rows
     auto issue_loads = [&](int g) {
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-#pragma unroll
-            for (int i = 0; i < XQ; ++i) {
-                const int m = mt * 16 + i * 4 + kq;
-                xv[mt][i] = u32x4{0u, 0u, 0u, 0u};
-                if (m < a.M && (!EXT || 128 * g + 8 * slot < a.k_valid))
-                    xv[mt][i] = *reinterpret_cast<const u32x4*>(a.X + (size_t)m * a.ldx + 128 * g + 8 * slot);
-            }
+        for (int i = 0; i < XQ; ++i) {
+            const int m = i * 4 + kq;
+            xv[i] = u32x4{0u, 0u, 0u, 0u};
+            if (m < a.M && (!EXT || 128 * g + 8 * slot < a.k_valid))
+                xv[i] = *reinterpret_cast<const u32x4*>(a.X + (size_t)m * a.ldx + 128 * g + 8 * slot);
         }
         if (!a.per_column) {
             sc = *reinterpret_cast<const u32x4*>(strip_s + (size_t)g * a.N + scale_off);
@@ -168,43 +160,40 @@ void w4a16_stream_kernel(const StreamArgs a) {
         issue_loads(g);
         // ---- rotate (optionally) and stage the activations in LDS ------------------
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
-#pragma unroll
-            for (int i = 0; i < XQ; ++i) {
-                const int mrow = mt * 16 + i * 4;
-                if (mrow < a.xrows) {  // uniform
-                    u32x4 v = xv[mt][i];
-                    if (HAD) {
-                        float f[8];
-#pragma unroll
-                        for (int p = 0; p < 4; ++p) {
-                            const h2 hv = bits_to_h2(v[p]);
-                            f[2 * p] = (float)hv.x;
-                            f[2 * p + 1] = (float)hv.y;
-                        }
-                        wht128_row16(f, slot);
-#pragma unroll
-                        for (int p = 0; p < 4; ++p) {
-                            h2 hv;
-                            hv.x = scaled_to_half(f[2 * p], a.had_scale);
-                            hv.y = scaled_to_half(f[2 * p + 1], a.had_scale);
-                            v[p] = h2_to_bits(hv);
-                        }
-                    }
-                    // 8 * 2^-24 * (sum of the row), from the values the MFMA will see
-                    float sum = 0.f;
+        for (int i = 0; i < XQ; ++i) {
+            const int mrow = i * 4;
+            if (mrow < a.xrows) {  // uniform
+                u32x4 v = xv[i];
+                if (HAD) {
+                    float f[8];
 #pragma unroll
                     for (int p = 0; p < 4; ++p) {
                         const h2 hv = bits_to_h2(v[p]);
-                        sum += (float)hv.x + (float)hv.y;
+                        f[2 * p] = (float)hv.x;
+                        f[2 * p + 1] = (float)hv.y;
                     }
+                    wht128_row16(f, slot);
 #pragma unroll
-                    for (int d = 1; d < 16; d <<= 1) sum += __shfl_xor(sum, d, kWave);
-                    uint32_t* row = xs + (size_t)(mrow + kq) * kXsStride;
-#pragma unroll
-                    for (int p = 0; p < 4; ++p) row[stage_off + 4 * p] = h2_to_bits(bits_to_h2(v[p]) * stage_mul2);
-                    if (slot == 0) reinterpret_cast<float*>(row)[64] = sum * (8.0f / kAccumScale);
+                    for (int p = 0; p < 4; ++p) {
+                        h2 hv;
+                        hv.x = scaled_to_half(f[2 * p], a.had_scale);
+                        hv.y = scaled_to_half(f[2 * p + 1], a.had_scale);
+                        v[p] = h2_to_bits(hv);
+                    }
                 }
+                // 8 * 2^-24 * (sum of the row), from the values the MFMA will see
+                float sum = 0.f;
+#pragma unroll
+                for (int p = 0; p < 4; ++p) {
+                    const h2 hv = bits_to_h2(v[p]);
+                    sum += (float)hv.x + (float)hv.y;
+                }
+#pragma unroll
+                for (int d = 1; d < 16; d <<= 1) sum += __shfl_xor(sum, d, kWave);
+                uint32_t* row = xs + (size_t)(mrow + kq) * kXsStride;
+#pragma unroll
+                for (int p = 0; p < 4; ++p) row[stage_off + 4 * p] = h2_to_bits(bits_to_h2(v[p]) * stage_mul2);
+                if (slot == 0) reinterpret_cast<float*>(row)[64] = sum * (8.0f / kAccumScale);
             }
         }
         // LDS operations of one wave complete in issue order: the reads below see
@@ -215,26 +204,23 @@ void w4a16_stream_kernel(const StreamArgs a) {
 
         const u32x4 (&cur)[2 * RPW] = wq;
         const u32x4 sc_cur = sc;
-        h8 xa[RPW][MT];
-        f4 zp[MT];  // minus 8 * row sums for this lane's four output rows: the first MFMA's C operand
+        h8 xa[RPW];
+        f4 zp;  // minus 8 * row sums for this lane's four output rows: the first MFMA's C operand
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) {
+        for (int rp = 0; rp < RPW; ++rp)
+            xa[rp] = __builtin_bit_cast(h8, *reinterpret_cast<const u32x4*>(xs + xrow_of + 16 * rp));
 #pragma unroll
-            for (int rp = 0; rp < RPW; ++rp)
-                xa[rp][mt] = __builtin_bit_cast(h8, *reinterpret_cast<const u32x4*>(xs + xrow_of[mt] + 16 * rp));
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int r = mt * 16 + 4 * kq + v;
-                const float* sums = reinterpret_cast<const float*>(xs) + (r < a.xrows ? r : a.xrows - 1) * kXsStride + 64;
-                zp[mt][v] = (v >= NV) ? 0.f : -sums[0];
-            }
+        for (int v = 0; v < 4; ++v) {
+            const int r = 4 * kq + v;
+            const float* sums = reinterpret_cast<const float*>(xs) + (r < a.xrows ? r : a.xrows - 1) * kXsStride + 64;
+            zp[v] = (v >= NV) ? 0.f : -sums[0];
         }
         // two passes over the columns (word pairs j) keep the group's raw dot products in
         // sixteen registers; the scale of output column jb of this lane is half jb of the
         // 16-byte scale load
 #pragma unroll
         for (int jh = 0; jh < 2; ++jh) {
-            f4 dot[MT][4];
+            f4 dot[4];
 #pragma unroll
             for (int rp = 0; rp < RPW; ++rp) {
 #pragma unroll
@@ -247,10 +233,8 @@ void w4a16_stream_kernel(const StreamArgs a) {
                         const uint32_t p1 = blk ? (q1 >> 8) : q1;
                         const u32x4 raw = u32x4{p0 & mask_low, p0 & mask_high, p1 & mask_low, p1 & mask_high};
                         const h8 bw = __builtin_bit_cast(h8, raw);
-#pragma unroll
-                        for (int mt = 0; mt < MT; ++mt)
-                            dot[mt][2 * jl + blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                                xa[rp][mt], bw, rp == 0 ? zp[mt] : dot[mt][2 * jl + blk], 0, 0, 0);
+                        dot[2 * jl + blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
+                            xa[rp], bw, rp == 0 ? zp : dot[2 * jl + blk], 0, 0, 0);
                     }
                 }
             }
@@ -260,15 +244,13 @@ void w4a16_stream_kernel(const StreamArgs a) {
                 const h2 pr = bits_to_h2(sc_cur[jb >> 1]);
                 const float sf = (float)((jb & 1) ? pr.y : pr.x);
 #pragma unroll
-                for (int mt = 0; mt < MT; ++mt)
-#pragma unroll
-                    for (int v = 0; v < NV; ++v) acc[mt][jb][v] += dot[mt][jq][v] * sf;
+                for (int v = 0; v < NV; ++v) acc[jb][v] += dot[jq][v] * sf;
             }
         }
     }
 
     // ---- combine the waves (fixed order), then the K splits ------------------------------
-    // acc[mt][jb][v] on lane l is row m = 16 mt + 4 (l/16) + v, column
+    // acc[jb][v] on lane l is row m = 4 (l/16) + v, column
     // 128 strip + 64 (slot/8) + 16 (jb/2) + 8 (jb%2) + slot%8.
     // The exchange area follows the staging rows, so no barrier is needed before the first
     // round.  With at most four activation rows all waves fit one round.
@@ -283,66 +265,63 @@ void w4a16_stream_kernel(const StreamArgs a) {
     const bool gated = EXT && a.epi.gated != 0;  // uniform
     const int col_pair = col_out ^ 64;    // the other half of a (gate, up) pair
     bool first_round = true;
-    for (int mt = 0; mt < MT; ++mt) {
-        if (mt * 16 >= a.M) break;
-        float tot[NI], oth[NI];
+    float tot[NI], oth[NI];
 #pragma unroll
-        for (int i = 0; i < NI; ++i) tot[i] = oth[i] = 0.f;
-        for (int round = 0; round < WAVES / wpr; ++round) {
-            if (!first_round) __syncthreads();
-            first_round = false;
-            if (w / wpr == round) {
+    for (int i = 0; i < NI; ++i) tot[i] = oth[i] = 0.f;
+    for (int round = 0; round < WAVES / wpr; ++round) {
+        if (!first_round) __syncthreads();
+        first_round = false;
+        if (w / wpr == round) {
 #pragma unroll
-                for (int jb = 0; jb < 8; ++jb) {
+            for (int jb = 0; jb < 8; ++jb) {
 #pragma unroll
-                    for (int v = 0; v < NV; ++v) {
-                        const int ml = 4 * kq + v;
-                        if (mt * 16 + ml < a.M)
-                            red[((w % wpr) * rr_rows + ml) * 128 + ncol_lane + 16 * (jb >> 1) + 8 * (jb & 1)] =
-                                acc[mt][jb][v] * kAccumScale;
-                    }
-                }
-            }
-            __syncthreads();
-#pragma unroll
-            for (int i = 0; i < NI; ++i) {
-                const int ml = (tid >> 7) + RPT * i;
-                if (mt * 16 + ml < a.M) {
-                    for (int ww = 0; ww < wpr; ++ww) {
-                        tot[i] += red[(ww * rr_rows + ml) * 128 + col_out];
-                        if (gated) oth[i] += red[(ww * rr_rows + ml) * 128 + col_pair];
-                    }
+                for (int v = 0; v < NV; ++v) {
+                    const int ml = 4 * kq + v;
+                    if (ml < a.M)
+                        red[((w % wpr) * rr_rows + ml) * 128 + ncol_lane + 16 * (jb >> 1) + 8 * (jb & 1)] =
+                            acc[jb][v] * kAccumScale;
                 }
             }
         }
+        __syncthreads();
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int m = mt * 16 + (tid >> 7) + RPT * i;
-            if (m >= a.M) continue;
-            unsigned long long* word = a.accum + (size_t)m * a.N + n_out;
-            if (!gated) {
-                float total = tot[i];
-                const bool mine = a.splits == 1 || accum_add(word, tot[i], a.splits, total);
-                if (mine) {
-                    if constexpr (EXT) {
-                        finish_store(a.epi, a.D, m, n_out, total);
-                    } else if (a.epi.out_f32) {
-                        reinterpret_cast<float*>(a.D)[(size_t)m * a.N + n_out] = total;
-                    } else {
-                        reinterpret_cast<half_t*>(a.D)[(size_t)m * a.N + n_out] = (half_t)total;
-                    }
-                    if (a.splits != 1) accum_reset(word);
+            const int ml = (tid >> 7) + RPT * i;
+            if (ml < a.M) {
+                for (int ww = 0; ww < wpr; ++ww) {
+                    tot[i] += red[(ww * rr_rows + ml) * 128 + col_out];
+                    if (gated) oth[i] += red[(ww * rr_rows + ml) * 128 + col_pair];
                 }
-            } else if (col_out < 64) {
-                const int n_pair = 64 * strip + col_out;
-                if (a.splits == 1) {
-                    finish_store_gated(a.epi, a.D, m, n_pair, tot[i], oth[i]);
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+        const int m = (tid >> 7) + RPT * i;
+        if (m >= a.M) continue;
+        unsigned long long* word = a.accum + (size_t)m * a.N + n_out;
+        if (!gated) {
+            float total = tot[i];
+            const bool mine = a.splits == 1 || accum_add(word, tot[i], a.splits, total);
+            if (mine) {
+                if constexpr (EXT) {
+                    finish_store(a.epi, a.D, m, n_out, total);
+                } else if (a.epi.out_f32) {
+                    reinterpret_cast<float*>(a.D)[(size_t)m * a.N + n_out] = total;
                 } else {
-                    float total_g, total_u;
-                    if (accum_add_pair(word, word + 64, tot[i], oth[i], a.splits, total_g, total_u)) {
-                        finish_store_gated(a.epi, a.D, m, n_pair, total_g, total_u);
-                        accum_reset(word);
-                    }
+                    reinterpret_cast<half_t*>(a.D)[(size_t)m * a.N + n_out] = (half_t)total;
+                }
+                if (a.splits != 1) accum_reset(word);
+            }
+        } else if (col_out < 64) {
+            const int n_pair = 64 * strip + col_out;
+            if (a.splits == 1) {
+                finish_store_gated(a.epi, a.D, m, n_pair, tot[i], oth[i]);
+            } else {
+                float total_g, total_u;
+                if (accum_add_pair(word, word + 64, tot[i], oth[i], a.splits, total_g, total_u)) {
+                    finish_store_gated(a.epi, a.D, m, n_pair, total_g, total_u);
+                    accum_reset(word);
                 }
             }
         }
@@ -399,19 +378,19 @@ static StreamPlan stream_plan(int m, int n, int k, int upw_override, int waves_o
 }
 
 size_t stream_accum_bytes(int m, int n, int k) {
-    // one 64-bit word per output element of a 64-row slab, whenever some plan splits K
+    // one 64-bit word per output element of a 16-row slab, whenever some plan splits K
     const int G = k / 128;
     if (G <= 4) return 0;
-    const int mrows = m < 64 ? m : 64;
+    const int mrows = m < 16 ? m : 16;
     return (size_t)mrows * n * sizeof(unsigned long long);
 }
 
-template <int MT, int RC, bool HAD, int WAVES, bool EXT>
+template <int RC, bool HAD, int WAVES, bool EXT>
 static hipError_t launch_one(const StreamArgs& a, hipStream_t stream) {
     const size_t stage = (size_t)WAVES * a.xrows * kXsStride * 4;
     const size_t red = a.xrows <= 4 ? (size_t)WAVES * 4 * 128 * 4 : (size_t)4 * 16 * 128 * 4;
     const size_t shmem = stage + red;
-    auto kern = &w4a16_stream_kernel<MT, RC, HAD, WAVES, EXT>;
+    auto kern = &w4a16_stream_kernel<RC, HAD, WAVES, EXT>;
     if (shmem > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
@@ -422,32 +401,25 @@ static hipError_t launch_one(const StreamArgs& a, hipStream_t stream) {
     return hipGetLastError();
 }
 
-// The plain instantiation exists for the decode shapes (one 16-row tile); larger tiles are only
-// reached by forcing this kernel and always take the full one.
-template <int MT, int RC, bool HAD>
+template <int RC, bool HAD>
 static hipError_t launch_waves(const StreamArgs& a, int waves, bool ext, hipStream_t stream) {
-    if constexpr (MT == 1) {
-        if (waves == 8)
-            return ext ? launch_one<MT, RC, HAD, 8, true>(a, stream) : launch_one<MT, RC, HAD, 8, false>(a, stream);
-        return ext ? launch_one<MT, RC, HAD, 4, true>(a, stream) : launch_one<MT, RC, HAD, 4, false>(a, stream);
-    }
-    return launch_one<MT, RC, HAD, 4, true>(a, stream);
+    if (waves == 8)
+        return ext ? launch_one<RC, HAD, 8, true>(a, stream) : launch_one<RC, HAD, 8, false>(a, stream);
+    return ext ? launch_one<RC, HAD, 4, true>(a, stream) : launch_one<RC, HAD, 4, false>(a, stream);
 }
 
 template <bool HAD>
-static hipError_t launch_rows(const StreamArgs& a, int mt, int waves, hipStream_t stream) {
+static hipError_t launch_rows(const StreamArgs& a, int waves, hipStream_t stream) {
     const Epilogue& e = a.epi;
     const bool ext = e.gated || e.bias || e.transpose || e.n_store != a.N || e.ldd != a.N || a.k_valid != a.K;
-    if (mt == 4) return launch_waves<4, 16, HAD>(a, waves, ext, stream);
-    if (mt == 2) return launch_waves<2, 16, HAD>(a, waves, ext, stream);
-    if (a.M == 1) return launch_waves<1, 1, HAD>(a, waves, ext, stream);
-    if (a.M == 2) return launch_waves<1, 2, HAD>(a, waves, ext, stream);
-    if (a.M <= 4) return launch_waves<1, 4, HAD>(a, waves, ext, stream);
-    if (a.M <= 8) return launch_waves<1, 8, HAD>(a, waves, ext, stream);
-    return launch_waves<1, 16, HAD>(a, waves, ext, stream);
+    if (a.M == 1) return launch_waves<1, HAD>(a, waves, ext, stream);
+    if (a.M == 2) return launch_waves<2, HAD>(a, waves, ext, stream);
+    if (a.M <= 4) return launch_waves<4, HAD>(a, waves, ext, stream);
+    if (a.M <= 8) return launch_waves<8, HAD>(a, waves, ext, stream);
+    return launch_waves<16, HAD>(a, waves, ext, stream);
 }
 
-// Rows are processed in slabs of at most 64; every slab re-streams the weights.
+// Rows are processed in slabs of at most 16; every slab re-streams the weights.
 // tune: bits 0..7 groups per wave, bits 8..12 waves per workgroup (4 or 8); zero fields mean
 // "choose".
 int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const void* S, void* D,
@@ -468,18 +440,16 @@ int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const 
     int waves_override = (int)((tune >> 8) & 0x1fu);
     if (waves_override != 4 && waves_override != 8) waves_override = 0;
     const size_t out_elt = epi.out_f32 ? 4 : 2;
-    for (int m0 = 0; m0 < m; m0 += 64) {
-        const int mm = (m - m0) < 64 ? (m - m0) : 64;
-        const int mt = mm <= 16 ? 1 : (mm <= 32 ? 2 : 4);
-        const StreamPlan plan = stream_plan(mm, n, k, (int)(tune & 0xffu), mt == 1 ? waves_override : 4);
+    for (int m0 = 0; m0 < m; m0 += 16) {
+        const int mm = (m - m0) < 16 ? (m - m0) : 16;
+        const StreamPlan plan = stream_plan(mm, n, k, (int)(tune & 0xffu), waves_override);
         a.upw = plan.upw;
         a.splits = plan.splits;
         a.M = mm;
-        a.xrows = mt == 1 ? ((mm + 3) / 4) * 4 : mt * 16;
+        a.xrows = ((mm + 3) / 4) * 4;
         a.X = reinterpret_cast<const half_t*>(A) + (size_t)m0 * lda;
         a.D = reinterpret_cast<char*>(D) + (size_t)m0 * (epi.transpose ? 1 : epi.ldd) * out_elt;
-        const hipError_t e = had128 ? launch_rows<true>(a, mt, plan.waves, stream)
-                                    : launch_rows<false>(a, mt, plan.waves, stream);
+        const hipError_t e = had128 ? launch_rows<true>(a, plan.waves, stream) : launch_rows<false>(a, plan.waves, stream);
         if (e != hipSuccess) return UNIQL_E_LAUNCH;
     }
     return UNIQL_OK;
