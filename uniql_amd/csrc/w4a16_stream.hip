@@ -253,10 +253,11 @@ void w4a16_stream_kernel(const StreamArgs a) {
     // acc[jb][v] on lane l is row m = 4 (l/16) + v, column
     // 128 strip + 64 (slot/8) + 16 (jb/2) + 8 (jb%2) + slot%8.
     // The exchange area follows the staging rows, so no barrier is needed before the first
-    // round.  With at most four activation rows all waves fit one round.
+    // round.
     float* red = reinterpret_cast<float*>(lds + (size_t)WAVES * a.xrows * kXsStride);
-    const int rr_rows = a.xrows <= 4 ? 4 : 16;      // rows per wave in the exchange area
-    const int wpr = a.xrows <= 4 ? WAVES : 4;       // waves per round
+    // the exchange area holds 64 rows of 128 floats: all waves at once up to 8 activation rows
+    const int rr_rows = a.xrows <= 4 ? 4 : (a.xrows <= 8 ? 8 : 16);  // rows per wave in the exchange area
+    const int wpr = 64 / rr_rows < WAVES ? 64 / rr_rows : WAVES;     // waves per round
     constexpr int RPT = WAVES / 2;                  // output rows covered per pass of the workgroup
     constexpr int NI = 16 / RPT;                    // passes needed for 16 rows
     const int ncol_lane = 64 * (slot >> 3) + c8;
@@ -388,7 +389,9 @@ size_t stream_accum_bytes(int m, int n, int k) {
 template <int RC, bool HAD, int WAVES, bool EXT>
 static hipError_t launch_one(const StreamArgs& a, hipStream_t stream) {
     const size_t stage = (size_t)WAVES * a.xrows * kXsStride * 4;
-    const size_t red = a.xrows <= 4 ? (size_t)WAVES * 4 * 128 * 4 : (size_t)4 * 16 * 128 * 4;
+    const int rr_rows = a.xrows <= 4 ? 4 : (a.xrows <= 8 ? 8 : 16);
+    const int wpr = 64 / rr_rows < WAVES ? 64 / rr_rows : WAVES;
+    const size_t red = (size_t)wpr * rr_rows * 128 * 4;
     const size_t shmem = stage + red;
     auto kern = &w4a16_stream_kernel<RC, HAD, WAVES, EXT>;
     if (shmem > 64 * 1024) {
