@@ -21,7 +21,7 @@ the tiled MFMA kernel (TFLOP/s = 2 M K N / time, against 2.5 PFLOP/s dense fp16)
 working directory) the per-shape tables: decode M in {1,2,4,8}, prefill M in {256,1024,4096},
 the pruned Llama shapes with the fused 128-block rotation, the Mamba2 shapes, the embedding
 gather, the standalone transform, the MLP front with the SiLU epilogue against the unfused
-sequence, a decoder layer's linears and glue as 5 against 10 launches, and the rotary kernel.
+sequence, a decoder layer's linears and glue as 5 against 12 launches, and the rotary kernel.
 """
 from __future__ import annotations
 
@@ -253,9 +253,10 @@ def sweep(dev, gen, out_path):
         torch.cuda.empty_cache()
 
     # The linears and glue of one Llama-3.1-8B decoder layer around attention, per token batch:
-    # the reference's call sequence (q, k, v, rotary, o, gate, up, silu, multiply, down: 10
-    # launches, all on this build's kernels) against the fused one (qkv, rotary, o, gate/up with the
-    # SiLU epilogue, down: 5 launches).  Attention itself is left out of both.
+    # the reference's call sequence (q, k, v, rotary, o, residual add, gate, up, silu, multiply, down,
+    # residual add: 12 launches, all on this build's kernels) against the fused one (qkv, rotary,
+    # o + residual, gate/up with the SiLU epilogue, down + residual: 5 launches).  Attention itself
+    # is left out of both.
     from uniql_amd import layout
     hid, nq, nkv, hd, inter = 4096, 32, 8, 128, 14336
     for m in (1, 8):
@@ -284,24 +285,24 @@ def sweep(dev, gen, out_path):
             k = lin(w["k"], x, nkv * hd, hid)
             v = lin(w["v"], x, nkv * hd, hid)
             ops.rope_indices_(q.view(1, m, nq, hd), k.view(1, m, nkv, hd), cos, sin, idx)
-            o = lin(w["o"], attn, hid, nq * hd)
+            o = x + lin(w["o"], attn, hid, nq * hd)
             h = torch.nn.functional.silu(lin(w["gate"], o, inter, hid)) * lin(w["up"], o, inter, hid)
-            return lin(w["down"], h, hid, inter), v
+            return o + lin(w["down"], h, hid, inter), v
 
         def fused(i):
             w = sets[i % copies]
             qkv = lin(w["qkv"], x, (nq + 2 * nkv) * hd, hid)
             q, k = qkv[:, :nq * hd], qkv[:, nq * hd:(nq + nkv) * hd]
             ops.rope_indices_(q.unflatten(1, (nq, hd)).unsqueeze(0), k.unflatten(1, (nkv, hd)).unsqueeze(0), cos, sin, idx)
-            o = lin(w["o"], attn, hid, nq * hd)
+            o = lin(w["o"], attn, hid, nq * hd, residual=x)
             h = lin(w["gate_up"], o, 2 * inter, hid, silu_mul=True)
-            return lin(w["down"], h, hid, inter), qkv
+            return lin(w["down"], h, hid, inter, residual=o), qkv
 
         sec_u, _ = time_graphs(unfused, copies, 200, 20)
         sec_f, _ = time_graphs(fused, copies, 200, 20)
         rows.append(dict(op="decoder_layer_linears_and_glue", m=m, us_fused=sec_f * 1e6, us_unfused=sec_u * 1e6,
-                         launches_fused=5, launches_unfused=10))
-        print("decoder layer (linears + rotary + MLP glue, no attention) M=%d: 5 launches %.2f us, 10 launches %.2f us"
+                         launches_fused=5, launches_unfused=12))
+        print("decoder layer (linears + rotary + MLP glue + residuals, no attention) M=%d: 5 launches %.2f us, 12 launches %.2f us"
               % (m, sec_f * 1e6, sec_u * 1e6), file=sys.stderr, flush=True)
         del sets
         torch.cuda.empty_cache()

@@ -102,7 +102,8 @@ int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, v
  * The whole forward of the reference's layer in one call, with the work around the product
  * done inside the kernels instead of by separate tensor operations:
  * W4A16B16O16Linear.forward (quantize/quant_linear_layers.py:92-114: pad the input to k,
- * product, drop the padded output columns, add the bias), and, with UNIQL_EPI_SILU_MUL,
+ * product, drop the padded output columns, add the bias), the decoder layer's
+ * `residual + layer(x)` (modeling/llama/llama_qblocks.py:182,188) and, with UNIQL_EPI_SILU_MUL,
  * the MLP's act_fn(gate_proj(x)) * up_proj(x) (modeling/llama/llama_qblocks.py:48-51).
  * Arguments as uniql_w4a16_gemm, plus:
  *   k_in      columns of A that exist (lda >= k_in, k_in % 8 == 0, k - 128 < k_in <= k); K rows
@@ -110,6 +111,9 @@ int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, v
  *   bias      device, fp16 [n_out] in natural column order, or NULL; added to the fp16-rounded
  *             product and rounded again, as the reference's `y + self.bias` does.  With
  *             UNIQL_EPI_SILU_MUL: [2 n_out], the gate biases followed by the up biases
+ *   residual  device, fp16 [m, ldr] (ldr >= n_out) or NULL: added to the rounded (and biased)
+ *             product and rounded again; may be the same memory as D (every element is read
+ *             by the thread that writes it); not with UNIQL_EPI_SILU_MUL
  *   D, ldd    output rows of ldd elements (ldd >= n_out); 16-byte stores are used when
  *             ldd % 8 == 0 and D is 16-byte aligned
  *   n_out     output columns that exist (the module's out_features); the rest of n is dropped
@@ -129,6 +133,7 @@ enum { UNIQL_EPI_NONE = 0, UNIQL_EPI_SILU_MUL = 1 };
 size_t uniql_w4a16_linear_temp_bytes(int m, int n, int k, int k_in, int had_block);
 
 int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, const void* S, const void* bias,
+                       const void* residual, int64_t ldr,
                        void* D, int64_t ldd, int n_out, int epilogue,
                        const int32_t* workspace, int64_t workspace_len,
                        void* accum, size_t accum_bytes, void* temp, size_t temp_bytes,

@@ -42,7 +42,7 @@ def test_host_only_entry_points(lib):
     # one 64-bit word per output element of a (<= 64 row) slab when K can be split
     assert lib.uniql_w4a16_gemm_accum_bytes(1, 4096, 4096) == 4096 * 8
     assert lib.uniql_w4a16_gemm_accum_bytes(100, 4096, 4096) == 100 * 4096 * 8
-    assert lib.uniql_w4a16_gemm_accum_bytes(4096, 4096, 4096) == 64 * 4096 * 8
+    assert lib.uniql_w4a16_gemm_accum_bytes(4096, 4096, 4096) == 16 * 4096 * 8
     assert lib.uniql_w4a16_gemm_accum_bytes(1, 4096, 512) == 0
     assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 8192) == 2 * 8192 * 2
     assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 128) == 2 * 8192 * 2
@@ -59,7 +59,8 @@ def test_argument_checks_need_no_gpu(lib):
     assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 1, 4096, 4096, 32, 0, 1.0, 0, None) == -1
     assert f(None, 4096, None, None, None, None, 0, None, 0, None, 0, 0, 4096, 4096, 32, 0, 1.0, 0, None) == 0
     g = lib.uniql_w4a16_linear
-    args = dict(A=None, lda=4096, k_in=4096, B=None, S=None, bias=None, D=None, ldd=4096, n_out=4096, epilogue=0,
+    args = dict(A=None, lda=4096, k_in=4096, B=None, S=None, bias=None, residual=None, ldr=0, D=None, ldd=4096,
+                n_out=4096, epilogue=0,
                 workspace=None, workspace_len=0, accum=None, accum_bytes=0, temp=None, temp_bytes=0, m=1, n=4096,
                 k=4096, groups=32, had_block=0, had_scale=1.0, flags=0, stream=None)
 

@@ -1,6 +1,7 @@
 """A pruned-Llama style decoder layer assembled twice from the same quantised layers: the
 reference's call sequence (one module call per projection, tensor operations in between) and
-the fused sequence (q/k/v in one launch, rotary kernel, gate/up with the SiLU epilogue).  The two
+the fused sequence (q/k/v in one launch, rotary kernel, gate/up with the SiLU epilogue, the residual
+additions inside o_proj's and down_proj's calls).  The two
 must agree, and the unfused one must agree with the oracle evaluated layer by layer."""
 import numpy as np
 import pytest
@@ -62,8 +63,8 @@ def layer_fused(F, x, cos, sin, idx):
     v = v.reshape(b, s, KV_HEADS, PRUNED_DIM).transpose(1, 2)
     q, k = apply_rotary_pos_emb_indices(q, k, cos, sin, idx)
     a = attention(q, k, v).transpose(1, 2).reshape(b, s, HEADS * PRUNED_DIM)
-    h = x + F["o"](a)
-    return h + F["down"](F["gate_up"](h))
+    h = F["o"](a, residual=x)
+    return F["down"](F["gate_up"](h), residual=h)
 
 
 @pytest.mark.parametrize("bias", [False, True])

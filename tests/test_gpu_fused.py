@@ -64,6 +64,36 @@ def test_cut_and_bias_equal_the_unfused_sequence(gpu, m, k, n, n_out):
         assert (diff <= 1e-4 * np.sqrt(k) + step).all()
 
 
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 100, 256])
+@pytest.mark.parametrize("k,n,n_out", [(256, 256, 200), (4096, 3584, 3456)])
+def test_residual_add_equals_the_unfused_sequence(gpu, m, k, n, n_out):
+    """the decoder layer's `residual + layer(x)`: bit-exact against torch's fp16 add of the layer's
+    output, with and without a bias, also in place (D = residual)"""
+    from uniql_amd import ops
+    p = make_linear_problem(m, k, n, seed=m + k)
+    x, b, s = to_gpu(p, gpu)
+    ws = workspace_for(n, gpu)
+    gen = torch.Generator().manual_seed(m)
+    res = torch.randn(m, n_out, generator=gen).half().to(gpu)
+    bias = torch.randn(n_out, generator=gen).half().to(gpu)
+    plain = ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out)
+    assert torch.equal(ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, residual=res), res + plain)
+    biased = ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, bias=bias)
+    assert torch.equal(ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, bias=bias, residual=res), res + biased)
+    # a residual that is a column range of a wider tensor, and the result written over it
+    wide = torch.randn(m, n_out + 24, generator=gen).half().to(gpu)
+    view = wide[:, 8:8 + n_out]
+    want = view + plain
+    ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, residual=view, out=view)
+    assert torch.equal(view, want)
+    y32 = ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, residual=res, out_f32=True)
+    p32 = ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, out_f32=True)
+    assert torch.equal(y32, p32 + res.float())
+    with pytest.raises(RuntimeError):
+        ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out // 2, residual=res[:, :n_out // 2], silu_mul=True)
+    assert accumulators_are_zero()
+
+
 @pytest.mark.parametrize("m", [1, 5, 16, 40, 130])
 @pytest.mark.parametrize("k_in", [200, 248, 136])
 def test_input_padding_inside_the_call(gpu, m, k_in):

@@ -81,7 +81,8 @@ size_t uniql_w4a16_gemm_temp_bytes(int m, int n, int k, int had_block) {
 }
 
 int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, const void* S, const void* bias,
-                       void* D, int64_t ldd, int n_out, int epilogue, const int32_t* workspace,
+                       const void* residual, int64_t ldr, void* D, int64_t ldd, int n_out, int epilogue,
+                       const int32_t* workspace,
                        int64_t workspace_len, void* accum, size_t accum_bytes, void* temp, size_t temp_bytes, int m,
                        int n, int k, int groups, int had_block, float had_scale, unsigned flags, void* stream) {
     const int rc = check_linear_shape(m, n, k, groups);
@@ -98,6 +99,11 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
     if (!aligned16(A) || !aligned16(B) || !aligned16(S)) return UNIQL_E_ALIGN;
     if (reinterpret_cast<uintptr_t>(D) % (out_f32 ? 4 : 2) != 0) return UNIQL_E_ALIGN;
     if (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)) return UNIQL_E_ALIGN;
+    if (residual) {
+        if (gated) return UNIQL_E_UNSUPPORTED;
+        if (ldr < n_out) return UNIQL_E_SHAPE;
+        if (reinterpret_cast<uintptr_t>(residual) & 1u) return UNIQL_E_ALIGN;
+    }
     if (workspace && workspace_len < n / 128) return UNIQL_E_WORKSPACE;
     if (had_block != 0 && (!is_pow2(had_block) || had_block < 2 || had_block > 32768 || k % had_block != 0))
         return UNIQL_E_SHAPE;
@@ -145,6 +151,8 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
     }
     Epilogue epi;
     epi.bias = reinterpret_cast<const half_t*>(bias);
+    epi.residual = reinterpret_cast<const half_t*>(residual);
+    epi.ldr = ldr;
     epi.ldd = ldd;
     epi.n_store = n_out;
     epi.gated = gated ? 1 : 0;
@@ -164,7 +172,7 @@ int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, v
     // transposed: D is [n, m8] with m8 = m rounded up to 8, as the reference allocates it
     // (marlin_gemm_kernel.cuh:1023-1026)
     const int64_t ldd = (flags & UNIQL_F_TRANSPOSE_OUT) ? (int64_t)((m + 7) / 8) * 8 : n;
-    return uniql_w4a16_linear(A, lda, k, B, S, nullptr, D, ldd, n, UNIQL_EPI_NONE, workspace, workspace_len, accum,
+    return uniql_w4a16_linear(A, lda, k, B, S, nullptr, nullptr, 0, D, ldd, n, UNIQL_EPI_NONE, workspace, workspace_len, accum,
                               accum_bytes, temp, temp_bytes, m, n, k, groups, had_block, had_scale, flags, stream);
 }
 

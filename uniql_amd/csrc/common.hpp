@@ -82,10 +82,13 @@ __device__ __forceinline__ int single_scale_pos(int n) {
 // ---- what happens to a finished output element --------------------------------------
 // The reference's layer rounds the product to fp16, drops the padding columns, then adds the
 // fp16 bias (second rounding); its MLP applies SiLU to the fp16 gate output (third rounding)
-// and multiplies by the fp16 up output (fourth).  The same roundings are made here, in
+// and multiplies by the fp16 up output (fourth); its decoder layer adds the layer's fp16 output
+// to the fp16 residual stream (one more rounding).  The same roundings are made here, in
 // registers, so that the fused result equals the unfused sequence.
 struct Epilogue {
     const half_t* bias;  // natural order [n_store] (gated: gate biases, then up biases), or nullptr
+    const half_t* residual;  // [M][ldr], added to the rounded (and biased) product, or nullptr
+    int64_t ldr;
     int64_t ldd;         // elements between output rows
     int n_store;         // output columns that exist; columns from here on are dropped
     int gated;           // 1: columns c and c + 64 of a 128-column strip are the gate and up values
@@ -103,13 +106,15 @@ struct Epilogue {
 __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)); }
 
 // value of output column n (< n_store) from its fp32 product, and of a gated pair
-__device__ __forceinline__ half_t finish_half(const Epilogue& e, int n, float v) {
+__device__ __forceinline__ half_t finish_half(const Epilogue& e, int m, int n, float v) {
     half_t y = (half_t)v;
     if (e.bias) y = (half_t)((float)y + (float)e.bias[n]);
+    if (e.residual) y = (half_t)((float)e.residual[(size_t)m * e.ldr + n] + (float)y);
     return y;
 }
 __device__ __forceinline__ half_t finish_half_gated(const Epilogue& e, int n, float g, float u) {
-    const half_t g16 = finish_half(e, n, g);
+    half_t g16 = (half_t)g;
+    if (e.bias) g16 = (half_t)((float)g16 + (float)e.bias[n]);
     half_t u16 = (half_t)u;
     if (e.bias) u16 = (half_t)((float)u16 + (float)e.bias[e.n_store + n]);
     const half_t a16 = (half_t)silu_f32((float)g16);
@@ -119,10 +124,13 @@ __device__ __forceinline__ half_t finish_half_gated(const Epilogue& e, int n, fl
 __device__ __forceinline__ void finish_store(const Epilogue& e, void* D, int m, int n, float v) {
     if (n >= e.n_store) return;
     const size_t o = e.offset(m, n);
-    if (e.out_f32)
-        reinterpret_cast<float*>(D)[o] = e.bias ? v + (float)e.bias[n] : v;
-    else
-        reinterpret_cast<half_t*>(D)[o] = finish_half(e, n, v);
+    if (e.out_f32) {
+        if (e.bias) v += (float)e.bias[n];
+        if (e.residual) v += (float)e.residual[(size_t)m * e.ldr + n];
+        reinterpret_cast<float*>(D)[o] = v;
+    } else {
+        reinterpret_cast<half_t*>(D)[o] = finish_half(e, m, n, v);
+    }
 }
 
 __device__ __forceinline__ void finish_store_gated(const Epilogue& e, void* D, int m, int n, float g, float u) {

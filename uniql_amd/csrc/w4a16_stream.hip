@@ -414,7 +414,8 @@ static hipError_t launch_waves(const StreamArgs& a, int waves, bool ext, hipStre
 template <bool HAD>
 static hipError_t launch_rows(const StreamArgs& a, int waves, hipStream_t stream) {
     const Epilogue& e = a.epi;
-    const bool ext = e.gated || e.bias || e.transpose || e.n_store != a.N || e.ldd != a.N || a.k_valid != a.K;
+    const bool ext = e.gated || e.bias || e.residual || e.transpose || e.n_store != a.N || e.ldd != a.N ||
+                     a.k_valid != a.K;
     if (a.M == 1) return launch_waves<1, HAD>(a, waves, ext, stream);
     if (a.M == 2) return launch_waves<2, HAD>(a, waves, ext, stream);
     if (a.M <= 4) return launch_waves<4, HAD>(a, waves, ext, stream);
@@ -452,6 +453,7 @@ int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const 
         a.xrows = ((mm + 3) / 4) * 4;
         a.X = reinterpret_cast<const half_t*>(A) + (size_t)m0 * lda;
         a.D = reinterpret_cast<char*>(D) + (size_t)m0 * (epi.transpose ? 1 : epi.ldd) * out_elt;
+        if (epi.residual) a.epi.residual = epi.residual + (size_t)m0 * epi.ldr;
         const hipError_t e = had128 ? launch_rows<true>(a, plan.waves, stream) : launch_rows<false>(a, plan.waves, stream);
         if (e != hipSuccess) return UNIQL_E_LAUNCH;
     }

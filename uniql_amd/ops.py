@@ -107,11 +107,12 @@ def w4a16_gemm_ex(A: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: 
 
 def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: torch.Tensor, size_n: int,
                  size_k: int, *, out_features: int | None = None, bias: torch.Tensor | None = None,
-                 silu_mul: bool = False, had_block: int = 0, had_scale: float = 1.0, out_f32: bool = False,
+                 residual: torch.Tensor | None = None, silu_mul: bool = False, had_block: int = 0, had_scale: float = 1.0, out_f32: bool = False,
                  out: torch.Tensor | None = None, flags: int = 0) -> torch.Tensor:
     """The layer's whole forward in one call (uniql_w4a16_linear): x [m, in_features] with
     in_features <= size_k (the kernel pads), product with the packed weights, only the first
-    `out_features` columns stored, `bias` added with the reference's rounding.  With
+    `out_features` columns stored, `bias` and then `residual` ([m, out_features], the decoder
+    layer's `residual + layer(x)`) added with the reference's roundings.  With
     `silu_mul` the packed tensors hold a gate and an up projection interleaved in 64-column
     blocks (layout.interleave_gate_up) and the result is silu(gate) * up, [m, out_features].
     `out`: optional destination, a 2-D view with unit inner stride (for example a column range
@@ -139,6 +140,12 @@ def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: t
         _require_gpu(bias, "bias")
         if bias.dtype != torch.float16 or not bias.is_contiguous() or bias.numel() != (2 if silu_mul else 1) * n_out:
             raise RuntimeError("bias must be contiguous float16 with one entry per output column")
+    if residual is not None:
+        _require_gpu(residual, "residual")
+        if silu_mul:
+            raise RuntimeError("a residual cannot be combined with the gated epilogue")
+        if residual.dtype != torch.float16 or tuple(residual.shape) != (m, n_out) or residual.stride(1) != 1:
+            raise RuntimeError("residual must be float16 [m, out_features] with unit inner stride")
     if k_in % 8 or (m > 1 and x.stride(0) % 8) or x.data_ptr() % 16:
         # rare: rows that cannot be read in 16-byte pieces are copied (and padded) here
         x = torch.nn.functional.pad(x, (0, size_k - k_in))
@@ -163,6 +170,8 @@ def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: t
         ldd = out.stride(0) if m > 1 else n_out
         code = lib.uniql_w4a16_linear(
             x.data_ptr(), lda, k_in, B.data_ptr(), s.data_ptr(), bias.data_ptr() if bias is not None else None,
+            residual.data_ptr() if residual is not None else None,
+            (residual.stride(0) if m > 1 else n_out) if residual is not None else 0,
             out.data_ptr(), ldd, n_out, _capi.EPI_SILU_MUL if silu_mul else _capi.EPI_NONE,
             workspace.data_ptr(), workspace.numel(),
             accum.data_ptr() if accum is not None else None, accum.numel() * 8 if accum is not None else 0,

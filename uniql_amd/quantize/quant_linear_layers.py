@@ -95,15 +95,18 @@ class W4A16B16O16Linear(nn.Module):
         return self
 
     @torch.no_grad()
-    def forward(self, x):
+    def forward(self, x, residual=None):
         """Padding of the input, the product, the cut of the padded output columns and the bias
-        (quant_linear_layers.py:92-114) happen inside one kernel call."""
+        (quant_linear_layers.py:92-114) happen inside one kernel call.  Beyond the reference:
+        `residual` (same shape as the result) is added in the same call, with the rounding of
+        the decoder layer's `residual + layer(x)`."""
         lead = x.shape[:-1]
         x2 = x.reshape(-1, x.shape[-1])
         if x2.stride(-1) != 1:
             x2 = x2.contiguous()
         y = ops.w4a16_linear(x2, self.weight, self.scale, self.workspace, self.size_n, self.size_k,
                              out_features=self.out_features, bias=None if self.bias is None else self.bias.data,
+                             residual=None if residual is None else residual.reshape(-1, self.out_features),
                              had_block=self.had_block, had_scale=self.had_scale)
         return y.view(*lead, self.out_features)
 
