@@ -11,7 +11,7 @@
 //
 // Every byte of the 1 KiB row segment is fetched once and eight MFMAs (one per jb)
 // consume two packed rows (32 K values) at a time.  The activations are the A operand:
-// rows of X (up to 16 per M-tile) staged through LDS in the same K order.  MFMA is
+// rows of X (up to 16 per launch) staged through LDS in the same K order.  MFMA is
 // used purely as a wide dot-product unit: its cost does not depend on M, so
 // M = 1..16 all run at the weight-streaming rate.
 //
@@ -31,7 +31,7 @@
 // the same value as the reference's up to its fp16 rounding of every scaled weight.
 //
 // Work split: unit = (strip of 128 columns) x (group of 128 K).  A wave owns `upw`
-// consecutive groups of a strip, the four waves of a workgroup own consecutive
+// consecutive groups of a strip, the four or eight waves of a workgroup own consecutive
 // group ranges, partial sums meet in LDS.  When K is split over several workgroups,
 // each output element has a 64-bit word in a zero-initialised accumulator: bits 8..63
 // hold the running sum as a fixed-point integer (2^-24 units), bits 0..7 the number of
