@@ -224,6 +224,7 @@ int uniql_w4_embedding_quantize(const void* W, int64_t ldw, void* packed, void* 
  *   indices  device, [n_kv_heads, head_dim] integers of index_bytes (1: uint8 as the module
  *            stores them, 4: int32, 8: int64), each < cos_dim; query head h uses row
  *            h / (n_q_heads / n_kv_heads)
+ * rows = 0 (with any seq_len >= 0) is a valid call that does nothing.
  */
 int uniql_rope_indices(void* q, int64_t q_row_stride, void* k, int64_t k_row_stride,
                        const void* cos, const void* sin, int64_t cos_row_stride,

@@ -121,3 +121,44 @@ def test_extension_aliases_and_graph_capture(gpu):
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
     check_layer_output(out.cpu().numpy(), reference_product(p))
+
+
+def test_empty_inputs(gpu):
+    """Zero tokens go through every module without a launch and give correctly shaped, empty
+    results (a batch whose sequences have all finished, an empty id list)."""
+    from uniql_amd.quantize.quant_linear_layers import W4A16B16O16Linear
+    from uniql_amd.quantize.quant_embedding_layers import W4O16Embedding
+    from uniql_amd.quantize.quant_hadamard_layers import Hadamard
+    from uniql_amd.quantize.fused_layers import W4A16FusedLinear, W4A16GateUpSiLU
+    from uniql_amd import ops
+
+    q = W4A16B16O16Linear.from_fp16(make_linear(200, 300, True, 3).to(gpu))
+    for shape in [(0, 200), (2, 0, 200), (0, 5, 200)]:
+        y = q(torch.empty(shape, dtype=torch.float16, device=gpu))
+        assert y.shape == (*shape[:-1], 300) and y.dtype == torch.float16
+    a = W4A16B16O16Linear.from_fp16(make_linear(256, 256, False, 4).to(gpu))
+    b = W4A16B16O16Linear.from_fp16(make_linear(256, 512, False, 5).to(gpu))
+    parts = W4A16FusedLinear.from_linears([a, b])(torch.empty(0, 256, dtype=torch.float16, device=gpu))
+    assert [tuple(p.shape) for p in parts] == [(0, 256), (0, 512)]
+    h = W4A16GateUpSiLU.from_linears(b, b)(torch.empty(3, 0, 256, dtype=torch.float16, device=gpu))
+    assert h.shape == (3, 0, 512)
+
+    emb = torch.nn.Embedding(64, 128).half().to(gpu)
+    e = W4O16Embedding.from_fp16(emb)
+    for shape in [(0,), (2, 0)]:
+        out = e(torch.empty(shape, dtype=torch.int64, device=gpu))
+        assert out.shape == (*shape, 128) and out.dtype == torch.float16
+
+    assert Hadamard(256).to(gpu)(torch.empty(0, 256, dtype=torch.float16, device=gpu)).shape == (0, 256)
+
+    qh = torch.empty(1, 0, 4, 64, dtype=torch.float16, device=gpu)
+    kh = torch.empty(1, 0, 2, 64, dtype=torch.float16, device=gpu)
+    cos = torch.empty(1, 0, 64, dtype=torch.float16, device=gpu)
+    idx = torch.arange(32, device=gpu, dtype=torch.int32).repeat(2, 1)
+    idx = torch.cat([idx, idx], dim=1).contiguous()
+    ops.rope_indices_(qh, kh, cos, cos.clone(), idx)
+
+    # the empty calls above leave later calls intact
+    x = torch.randn(2, 200).half().to(gpu)
+    assert torch.isfinite(q(x)).all()
+    torch.cuda.synchronize()

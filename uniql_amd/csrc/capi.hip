@@ -226,8 +226,9 @@ int uniql_rope_indices(void* q, int64_t q_row_stride, void* k, int64_t k_row_str
                        const void* sin, int64_t cos_row_stride, const void* indices, int index_bytes, int64_t rows,
                        int seq_len, int cos_batch, int n_q_heads, int n_kv_heads, int head_dim, int cos_dim,
                        void* stream) {
-    if (rows < 0 || seq_len <= 0 || n_q_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0 || cos_dim <= 0)
+    if (rows < 0 || seq_len < 0 || n_q_heads <= 0 || n_kv_heads <= 0 || head_dim <= 0 || cos_dim <= 0)
         return UNIQL_E_SHAPE;
+    if (seq_len == 0) return rows == 0 ? UNIQL_OK : UNIQL_E_SHAPE;  // no tokens: nothing to rotate
     if (head_dim % 2 != 0 || n_q_heads % n_kv_heads != 0) return UNIQL_E_SHAPE;
     if (index_bytes != 1 && index_bytes != 4 && index_bytes != 8) return UNIQL_E_UNSUPPORTED;
     if (index_bytes == 1 && cos_dim > 256) return UNIQL_E_SHAPE;
