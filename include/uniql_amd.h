@@ -51,6 +51,13 @@ enum {
 int uniql_abi_version(void);
 const char* uniql_status_string(int code);
 
+/* The identifier of the graph capture `stream` is recording into, 0 when it is not capturing.
+ * No counterpart in the reference (its wrapper allocates its scratch with torch on every call,
+ * csrc/linear/marlin_gemm_kernel.cuh:1018); a host shim that caches the zero-in / zero-out `accum`
+ * buffer needs it: a buffer allocated and zero-filled while capturing is only zero when that
+ * graph replays, so it must not serve another capture or eager calls. */
+int uniql_stream_capture_id(void* stream, unsigned long long* id);
+
 /*
  * D[m, n] = A[m, k] . dequant(B)[k, n],  fp16 in, fp32 accumulate, fp16 out.
  * Replaces quant_linear_cuda.w4a16o16_gemm (csrc/linear/quant_linear.cpp:6-24,

@@ -47,6 +47,7 @@ def test_host_only_entry_points(lib):
     assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 8192) == 2 * 8192 * 2
     assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 128) == 2 * 8192 * 2
     assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 0) == 0
+    assert lib.uniql_stream_capture_id(None, None) == -1    # the result pointer is checked before any HIP call
 
 
 def test_argument_checks_need_no_gpu(lib):

@@ -320,3 +320,68 @@ def test_side_stream_and_graph_replay(gpu):
             assert torch.equal(a, b)
     for buf in ops._accum_cache.values():
         assert int(buf.count_nonzero()) == 0
+
+
+def test_accumulator_cache_across_graphs_and_growth(gpu):
+    """The Python layer caches the zero-in / zero-out accumulator words per stream.  Two hazards:
+    a buffer allocated while a graph is being captured is only zero-filled when THAT graph
+    replays, so a second graph (replayed first) and eager calls must not depend on it; and a
+    buffer a graph has captured must stay allocated when a later, larger call replaces it."""
+    from uniql_amd import ops
+    ops.reset_accumulators()
+    small = make_linear_problem(1, 4096, 512, seed=311)       # K split with atomics, small accumulator
+    other = make_linear_problem(2, 2048, 256, seed=312)
+    large = make_linear_problem(48, 4096, 2048, seed=313)     # tiled kernel with K splits: more words
+    xs, bs, ss = to_gpu(small, gpu)
+    xo, bo, so = to_gpu(other, gpu)
+    xl, bl, sl = to_gpu(large, gpu)
+    ws_s, ws_o, ws_l = (workspace_for(p["n"], gpu) for p in (small, other, large))
+
+    def run_small():
+        return ops.w4a16_gemm_ex(xs, bs, ss, ws_s, 1, 512, 4096)
+
+    def run_other():
+        return ops.w4a16_gemm_ex(xo, bo, so, ws_o, 2, 256, 2048)
+
+    def run_large():
+        return ops.w4a16_gemm_ex(xl, bl, sl, ws_l, 48, 2048, 4096)
+
+    # first use of the capture stream happens inside the captures
+    g1, g2 = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g1):
+        y1 = run_small()
+    with torch.cuda.graph(g2):
+        y2 = run_other()
+    # dirty whatever the allocator hands out next, then replay the SECOND graph first
+    junk = [torch.full((1 << 18,), -1, dtype=torch.int64, device=gpu) for _ in range(8)]
+    del junk
+    g2.replay()
+    torch.cuda.synchronize()
+    want_small, want_other, want_large = run_small().clone(), run_other().clone(), run_large().clone()
+    assert torch.equal(y2, want_other)
+    g1.replay()
+    torch.cuda.synchronize()
+    assert torch.equal(y1, want_small)
+
+    # eager buffer captured by a graph, then outgrown by a larger call
+    ops.reset_accumulators()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        assert torch.equal(run_small(), want_small)           # sizes the side stream's buffer eagerly
+        g3 = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g3, stream=side):
+            y3 = run_small()
+        before = ops._accum_cache[(side.device.index, side.cuda_stream)]
+        assert torch.equal(run_large(), want_large)           # needs more words: the buffer is replaced
+        assert ops._accum_cache[(side.device.index, side.cuda_stream)] is not before
+        junk = [torch.full((1 << 16,), -1, dtype=torch.int64, device=gpu) for _ in range(16)]
+        for rep in range(2):
+            y3.fill_(float("nan"))
+            g3.replay()
+            side.synchronize()
+            assert torch.equal(y3, want_small), f"replay {rep}"
+        del junk
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    ops.reset_accumulators()

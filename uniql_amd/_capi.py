@@ -23,6 +23,7 @@ EPI_NONE, EPI_SILU_MUL = 0, 1
 SIGNATURES = {
     "uniql_abi_version": (c_int, []),
     "uniql_status_string": (c_char_p, [c_int]),
+    "uniql_stream_capture_id": (c_int, [c_void_p, ctypes.POINTER(ctypes.c_ulonglong)]),
     "uniql_w4a16_gemm_accum_bytes": (c_size_t, [c_int, c_int, c_int]),
     "uniql_w4a16_gemm_temp_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "uniql_w4a16_gemm": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p,

@@ -45,6 +45,16 @@ extern "C" {
 
 int uniql_abi_version(void) { return UNIQL_ABI_VERSION; }
 
+int uniql_stream_capture_id(void* stream, unsigned long long* id) {
+    if (!id) return UNIQL_E_NULL;
+    hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+    unsigned long long capture = 0;
+    if (hipStreamGetCaptureInfo(reinterpret_cast<hipStream_t>(stream), &status, &capture) != hipSuccess)
+        return UNIQL_E_LAUNCH;
+    *id = status == hipStreamCaptureStatusActive ? capture : 0;
+    return UNIQL_OK;
+}
+
 const char* uniql_status_string(int code) {
     switch (code) {
         case UNIQL_OK: return "ok";

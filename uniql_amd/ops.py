@@ -11,6 +11,8 @@ torch.cuda.graph capture.  Errors surface as RuntimeError.
 """
 from __future__ import annotations
 
+import ctypes
+
 import torch
 
 from . import _capi
@@ -30,21 +32,52 @@ def _stream_ptr(device: torch.device) -> int:
 # (device, stream): kernels on one stream run in order, so they can share it; work on
 # different streams may overlap and must not.
 _accum_cache: dict = {}
+# Buffers that were replaced by larger ones stay allocated: a captured graph may still hold
+# their address, and memory handed back to the allocator would be reused under it.
+_accum_retired: list = []
+# Buffers born inside a graph capture, keyed by the capture as well: their zero fill is a node
+# of that graph, so they are only known to be zero when that graph replays and serve nothing else.
+_accum_in_capture: dict = {}
+
+
+def _capture_id(stream_ptr: int) -> int:
+    out = ctypes.c_ulonglong(0)
+    _capi.check(_capi.load().uniql_stream_capture_id(stream_ptr, ctypes.byref(out)), "uniql_stream_capture_id")
+    return out.value
 
 
 def _accumulator(device: torch.device, nbytes: int) -> torch.Tensor:
-    key = (device.index, torch.cuda.current_stream(device).cuda_stream)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    key = (device.index, stream)
     buf = _accum_cache.get(key)
-    if buf is None or buf.numel() * 8 < nbytes:
-        buf = torch.zeros(max(nbytes // 8, 1 << 16), dtype=torch.int64, device=device)
-        _accum_cache[key] = buf
+    if buf is not None and buf.numel() * 8 >= nbytes:
+        return buf
+    words = max(nbytes // 8, 1 << 16)
+    capture = _capture_id(stream)
+    if capture:
+        ckey = (device.index, stream, capture)
+        cbuf = _accum_in_capture.get(ckey)
+        if cbuf is None or cbuf.numel() * 8 < nbytes:
+            if cbuf is not None:
+                _accum_retired.append(cbuf)
+            cbuf = torch.zeros(words, dtype=torch.int64, device=device)  # the fill is recorded in the graph
+            _accum_in_capture[ckey] = cbuf
+        return cbuf
+    if buf is not None:
+        _accum_retired.append(buf)
+        words = max(words, 2 * buf.numel())  # geometric growth bounds what retirement keeps
+    buf = torch.zeros(words, dtype=torch.int64, device=device)
+    _accum_cache[key] = buf
     return buf
 
 
 def reset_accumulators() -> None:
     """Drops the cached accumulator buffers (they are re-created zeroed).  Only needed
-    after a kernel was aborted half-way, which can leave non-zero words behind."""
+    after a kernel was aborted half-way, which can leave non-zero words behind.  Graphs
+    captured before the call hold the old buffers' addresses and must be captured again."""
     _accum_cache.clear()
+    _accum_retired.clear()
+    _accum_in_capture.clear()
 
 
 def _require_gpu(t: torch.Tensor, name: str) -> None:
