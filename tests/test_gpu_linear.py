@@ -359,9 +359,14 @@ def test_accumulator_cache_across_graphs_and_growth(gpu):
     torch.cuda.synchronize()
     want_small, want_other, want_large = run_small().clone(), run_other().clone(), run_large().clone()
     assert torch.equal(y2, want_other)
-    g1.replay()
-    torch.cuda.synchronize()
-    assert torch.equal(y1, want_small)
+    for rep in range(3):                                      # the recorded zero fills replay correctly too
+        y1.fill_(float("nan"))
+        y2.fill_(float("nan"))
+        g1.replay()
+        g2.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(y1, want_small) and torch.equal(y2, want_other), f"replay {rep}"
+        assert torch.equal(run_small(), want_small)           # eager work between the replays
 
     # eager buffer captured by a graph, then outgrown by a larger call
     ops.reset_accumulators()
