@@ -199,6 +199,25 @@ def test_row_stride(gpu):
     check_layer_output(y, reference_product(p))
 
 
+@pytest.mark.parametrize("m,had_block", [(3, 256), (3, 128), (40, 128), (40, 512)])
+def test_row_stride_with_rotation(gpu, m, had_block):
+    """A row-strided view whose rows are rotated first (not the 128-block rotation fused into the
+    streaming kernel, or any rotation ahead of the tiled kernel) gives the same bits as the
+    contiguous input."""
+    from uniql_amd import ops
+    p = make_linear_problem(m, 1024, 256, seed=60 + m)
+    x, b, s = to_gpu(p, gpu)
+    big = torch.full((m, 1536), 3.0, dtype=torch.float16, device=gpu)
+    big[:, :1024] = x
+    kw = dict(had_block=had_block, had_scale=had_block ** -0.5)
+    ws = workspace_for(256, gpu)
+    want = ops.w4a16_gemm_ex(x, b, s, ws, m, 256, 1024, **kw)
+    got = ops.w4a16_gemm_ex(big[:, :1024], b, s, ws, m, 256, 1024, **kw)
+    assert torch.equal(want, got)
+    xr = O.fwht(p["x"], had_block ** -0.5, block=had_block)
+    check_layer_output(got.cpu().numpy(), O.gemm_fp64(xr, O.dequant_codes(p["q"], p["s"])))
+
+
 # ------------------------------------------------------------------ fused rotation
 @pytest.mark.parametrize("m", [1, 5, 16, 40, 200])
 def test_fused_blockwise_hadamard(gpu, m):

@@ -10,7 +10,7 @@ size_t stream_accum_bytes(int m, int n, int k);
 int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, const Epilogue& epi, void* accum,
                 size_t accum_bytes, int m, int n, int k, int groups, unsigned tune, hipStream_t stream);
 int pad_rows_launch(const void* A, int64_t lda, int k_in, void* dst, int k, int m, hipStream_t stream);
-size_t tile_accum_bytes(int m, int n, int k);
+size_t tile_accum_bytes(int m, int n, int k, unsigned tune = 0);
 int dequant_launch(const void* B, const void* S, void* W, uint8_t* codes, int n, int k, int groups,
                    hipStream_t stream);
 int embedding_launch(const int64_t* ids, int64_t ntokens, const void* weight, const void* scales, void* out,
@@ -131,9 +131,16 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
     int k_valid = k_in;
     const bool had128 = (had_block == 128) && use_stream;
     const bool rotate_first = had_block != 0 && !had128;
-    const bool pad_first = k_in != k && (rotate_first || !use_stream);
+    // the transform kernel reads dense rows of k values: a strided or short input is first copied
+    // (and zero-padded) into the temporary buffer, then rotated there in place
+    const bool pad_first = rotate_first ? (k_in != k || lda != k) : (k_in != k && !use_stream);
     if (rotate_first || pad_first) {
         if (!temp || temp_bytes < round256((size_t)m * k * sizeof(half_t))) return UNIQL_E_WORKSPACE;
+    }
+    const unsigned tune = flags >> 8;  // tuning fields, see the header
+    if (!use_stream) {  // a forced number of K splits may need more words than the default plan
+        const size_t need = tile_accum_bytes(m, n, k, tune);
+        if (need > 0 && (!accum || accum_bytes < need)) return UNIQL_E_WORKSPACE;
     }
     if (pad_first) {
         const int e = pad_rows_launch(A, lda, k_in, temp, k, m, st);
@@ -143,19 +150,8 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
         k_valid = k;
     }
     if (rotate_first) {
-        // rotate into the temporary buffer (in place when the padded copy is already there),
-        // then run the plain product on it
-        if (ld != k) {
-            for (int r = 0; r < m; ++r) {
-                const int e = fwht_launch(reinterpret_cast<const half_t*>(Ain) + (size_t)r * ld,
-                                          reinterpret_cast<half_t*>(temp) + (size_t)r * k, 1, k, had_block, had_scale,
-                                          UNIQL_DT_F16, st);
-                if (e != UNIQL_OK) return e;
-            }
-        } else {
-            const int e = fwht_launch(Ain, temp, m, k, had_block, had_scale, UNIQL_DT_F16, st);
-            if (e != UNIQL_OK) return e;
-        }
+        const int e = fwht_launch(Ain, temp, m, k, had_block, had_scale, UNIQL_DT_F16, st);
+        if (e != UNIQL_OK) return e;
         Ain = temp;
         ld = k;
     }
@@ -169,7 +165,6 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
     epi.out_f32 = out_f32 ? 1 : 0;
     epi.transpose = transpose ? 1 : 0;
     epi.vec_ok = (!transpose && ldd % 8 == 0 && aligned16(D)) ? 1 : 0;
-    const unsigned tune = flags >> 8;  // tuning fields, see the header
     if (use_stream)
         return stream_launch(Ain, ld, k_valid, B, S, D, epi, accum, m, n, k, groups, had128, had_scale, tune, st);
     return tile_launch(Ain, ld, B, S, D, epi, accum, accum_bytes, m, n, k, groups, tune, st);

@@ -530,9 +530,11 @@ struct TilePlan {
 };
 static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_override = 0, int kw_override = 0);
 
-size_t tile_accum_bytes(int m, int n, int k) {
+// tune: the same fields as tile_launch takes
+size_t tile_accum_bytes(int m, int n, int k, unsigned tune) {
     // one word per output element, only when the plan splits K over workgroups
-    return tile_plan(m, n, k, 0).splits > 1 ? (size_t)m * n * sizeof(unsigned long long) : 0;
+    const TilePlan plan = tile_plan(m, n, k, (int)(tune & 0xffu), (int)((tune >> 8) & 0xfu), (int)((tune >> 12) & 0x3u));
+    return plan.splits > 1 ? (size_t)m * n * sizeof(unsigned long long) : 0;
 }
 
 // Measured on MI355X, in units of the time one MT = 4 workgroup takes for its K loop when every
