@@ -140,8 +140,9 @@ def w4a16_gemm_ex(A: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: 
 
 def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: torch.Tensor, size_n: int,
                  size_k: int, *, out_features: int | None = None, bias: torch.Tensor | None = None,
-                 residual: torch.Tensor | None = None, silu_mul: bool = False, had_block: int = 0, had_scale: float = 1.0, out_f32: bool = False,
-                 out: torch.Tensor | None = None, flags: int = 0) -> torch.Tensor:
+                 residual: torch.Tensor | None = None, silu_mul: bool = False, had_block: int = 0,
+                 had_scale: float = 1.0, out_f32: bool = False, out: torch.Tensor | None = None,
+                 flags: int = 0) -> torch.Tensor:
     """The layer's whole forward in one call (uniql_w4a16_linear): x [m, in_features] with
     in_features <= size_k (the kernel pads), product with the packed weights, only the first
     `out_features` columns stored, `bias` and then `residual` ([m, out_features], the decoder

@@ -2,8 +2,6 @@
 (reference: modeling/rope_triton.py, modeling/llama/llama_rope.py:38-96)."""
 from __future__ import annotations
 
-import torch
-
 from . import ops
 
 
