@@ -111,7 +111,10 @@ int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, v
  * W4A16B16O16Linear.forward (quantize/quant_linear_layers.py:92-114: pad the input to k,
  * product, drop the padded output columns, add the bias), the decoder layer's
  * `residual + layer(x)` (modeling/llama/llama_qblocks.py:182,188) and, with UNIQL_EPI_SILU_MUL,
- * the MLP's act_fn(gate_proj(x)) * up_proj(x) (modeling/llama/llama_qblocks.py:48-51).
+ * the MLP's act_fn(gate_proj(x)) * up_proj(x) (modeling/llama/llama_qblocks.py:48-51) or, with
+ * UNIQL_EPI_RELU2, the un-gated act_fn(up_proj(x)) with the squared ReLU
+ * (modeling/nemotron_h/nemotron_h_qblocks.py:577,588; mlp_hidden_act "relu2",
+ * modeling/nemotron_h/configuration_nemotron_h.py:145).
  * Arguments as uniql_w4a16_gemm, plus:
  *   k_in      columns of A that exist (lda >= k_in, k_in % 8 == 0, k - 128 < k_in <= k); K rows
  *             from k_in on count as zero activations (the module's pad_in)
@@ -120,7 +123,7 @@ int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, v
  *             UNIQL_EPI_SILU_MUL: [2 n_out], the gate biases followed by the up biases
  *   residual  device, fp16 [m, ldr] (ldr >= n_out) or NULL: added to the rounded (and biased)
  *             product and rounded again; may be the same memory as D (every element is read
- *             by the thread that writes it); not with UNIQL_EPI_SILU_MUL
+ *             by the thread that writes it); only with UNIQL_EPI_NONE
  *   D, ldd    output rows of ldd elements (ldd >= n_out); 16-byte stores are used when
  *             ldd % 8 == 0 and D is 16-byte aligned
  *   n_out     output columns that exist (the module's out_features); the rest of n is dropped
@@ -132,10 +135,12 @@ int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, v
  *             twice the padded width of one projection, n_out <= n/2, and
  *             D[m, j] = fp16(fp16(silu(g)) * u) with g, u the fp16-rounded (and biased) gate and
  *             up outputs of column j: the reference's sequence of roundings.
+ *             UNIQL_EPI_RELU2: D[m, j] = fp16(max(y, 0)^2) with y the fp16-rounded (and biased)
+ *             output: torch.square(relu(y)) on the fp16 tensor.
  *   temp      uniql_w4a16_linear_temp_bytes(m, n, k, k_in, had_block) bytes
  * With UNIQL_F_OUT_F32 D is float32 and no intermediate rounding is applied.
  */
-enum { UNIQL_EPI_NONE = 0, UNIQL_EPI_SILU_MUL = 1 };
+enum { UNIQL_EPI_NONE = 0, UNIQL_EPI_SILU_MUL = 1, UNIQL_EPI_RELU2 = 2 };
 
 size_t uniql_w4a16_linear_temp_bytes(int m, int n, int k, int k_in, int had_block);
 

@@ -22,9 +22,10 @@ Pinning status (what proves each function right, besides reading):
     brute-force; the reference module cannot be imported without its compiled
     extension, so `embedding_quantize`'s code selection at exact rounding ties
     is "parity unpinned" beyond those cases
-  * module forward with its fp16 roundings, SiLU-gated MLP front (linear_forward_fp16,
-    silu_fp16, mlp_gate_up) ................. torch's own fp16 CPU operators over all
-    finite fp16 inputs / random tensors (the reference calls exactly those operators)
+  * module forward with its fp16 roundings, SiLU-gated and squared-ReLU MLP fronts
+    (linear_forward_fp16, silu_fp16, mlp_gate_up, relu2_fp16) ... torch's own fp16 CPU
+    operators over all finite fp16 inputs / random tensors (the reference calls exactly
+    those operators)
   * rotary embedding with gathered frequencies (rope_indices) ... the textbook complex
     rotation in float64 for identity indices, an independently permuted frequency table,
     norm preservation, and torch's fp16 CPU arithmetic for the order of the roundings
@@ -300,6 +301,15 @@ def mlp_gate_up(gate16: np.ndarray, up16: np.ndarray) -> np.ndarray:
     a = silu_fp16(gate16).astype(np.float32)
     with np.errstate(over="ignore"):
         return (a * np.asarray(up16, dtype=np.float16).astype(np.float32)).astype(np.float16)
+
+
+def relu2_fp16(y16: np.ndarray) -> np.ndarray:
+    """act_fn(up_proj(x)) of the un-gated MLP with mlp_hidden_act = "relu2"
+    (nemotron_h_qblocks.py:577,588; transformers' ReLUSquaredActivation: relu, then
+    torch.square) on the layer's fp16 output: the exact square rounded once to fp16."""
+    r = np.maximum(np.asarray(y16, dtype=np.float16).astype(np.float32), np.float32(0.0))
+    with np.errstate(over="ignore"):
+        return (r * r).astype(np.float16)
 
 
 # --------------------------------------------------------------------------

@@ -74,7 +74,8 @@ def test_argument_checks_need_no_gpu(lib):
     assert call(n_out=4097) == -2
     assert call(epilogue=1, n_out=2049) == -2            # a gated call stores at most n/2 columns
     assert call(epilogue=1, n_out=2048, ldd=2048) == -1
-    assert call(epilogue=2) == -5
+    assert call(epilogue=2) == -1                        # squared ReLU: a known epilogue, pointers missing
+    assert call(epilogue=3) == -5
     assert call(ldd=4095) == -2
     assert call(flags=8, ldd=0) == -2                    # transposed: ldd counts rows
     assert call(m=0) == 0

@@ -276,6 +276,50 @@ def test_gate_up_module(gpu, in_f, width, bias):
         assert_close16(y.cpu().numpy(), t.cpu().numpy(), ulps=8, floor=floor, differing=5e-2)
 
 
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 100, 256])
+@pytest.mark.parametrize("k,n,n_out,bias", [(256, 256, 200, True), (4096, 3584, 3456, False), (1408, 512, 512, True)])
+def test_squared_relu_epilogue_equals_the_unfused_sequence(gpu, m, k, n, n_out, bias):
+    """act_fn(up_proj(x)) with the squared ReLU: bit-exact against the activation applied to the
+    layer's own output (torch's operators on the fp16 tensor, as the reference runs them), and
+    against the oracle's restatement on the same outputs."""
+    from transformers.activations import ACT2FN
+    from uniql_amd import ops
+    p = make_linear_problem(m, k, n, seed=m + k + n + 1)
+    x, b, s = to_gpu(p, gpu)
+    ws = workspace_for(n, gpu)
+    bias_t = torch.from_numpy(np.random.default_rng(6).standard_normal(n_out).astype(np.float16)).to(gpu) if bias else None
+    plain = ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, bias=bias_t)
+    got = ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, bias=bias_t, relu2=True)
+    assert torch.equal(got, ACT2FN["relu2"](plain))
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), O.relu2_fp16(plain.cpu().numpy()).view(np.uint16))
+    assert not torch.signbit(got).any()                               # negatives give +0, never -0
+    # fp32 output: the activation of the unrounded sum
+    plain32 = ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, bias=bias_t, out_f32=True)
+    got32 = ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, bias=bias_t, relu2=True, out_f32=True)
+    assert torch.equal(got32, torch.square(torch.relu(plain32)))
+    assert accumulators_are_zero()
+
+
+def test_squared_relu_mlp_module(gpu):
+    """The un-gated MLP of the squared-ReLU models: down_proj(act_fn(up_proj(x))) with the
+    activation inside the first layer's call (nemotron_h_qblocks.py:588)."""
+    from transformers.activations import ACT2FN
+    from uniql_amd.quantize.quant_linear_layers import W4A16B16O16Linear
+    g = torch.Generator().manual_seed(9)
+    up = torch.nn.Linear(512, 1408, bias=True).half()
+    down = torch.nn.Linear(1408, 512, bias=False).half()
+    for lin in (up, down):
+        lin.weight.data = (torch.randn(lin.weight.shape, generator=g) * 0.05).half()
+    up.bias.data = torch.randn(1408, generator=g).half()
+    qup, qdown = W4A16B16O16Linear.from_fp16(up.to(gpu)), W4A16B16O16Linear.from_fp16(down.to(gpu))
+    x = torch.randn(2, 5, 512, generator=g).half().to(gpu)
+    want = qdown(ACT2FN["relu2"](qup(x)))
+    got = qdown(qup(x, activation="relu2"))
+    assert got.shape == (2, 5, 512) and torch.equal(got, want)
+    with pytest.raises(ValueError):
+        qup(x, activation="gelu")
+
+
 def test_fused_call_errors(gpu):
     from uniql_amd import ops
     p = make_linear_problem(2, 256, 256)
@@ -291,3 +335,7 @@ def test_fused_call_errors(gpu):
         ops.w4a16_linear(x, b, s, ws, 256, 256, bias=torch.zeros(100, dtype=torch.float16, device=gpu))
     with pytest.raises(RuntimeError):
         ops.w4a16_linear(x, b, s, ws, 256, 256, out=torch.empty(2, 256, dtype=torch.float32, device=gpu))
+    with pytest.raises(RuntimeError):
+        ops.w4a16_linear(x, b, s, ws, 256, 256, out_features=128, silu_mul=True, relu2=True)
+    with pytest.raises(RuntimeError):
+        ops.w4a16_linear(x, b, s, ws, 256, 256, relu2=True, residual=torch.zeros(2, 256, dtype=torch.float16, device=gpu))

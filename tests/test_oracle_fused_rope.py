@@ -31,6 +31,19 @@ def test_silu_fp16_is_torchs_operator_on_every_finite_input():
     assert np.abs(O.silu_fp16(xs).astype(np.float64) - exact).max() < 2e-3
 
 
+def test_relu2_fp16_is_transformers_activation_on_every_finite_input():
+    """ACT2FN["relu2"] (relu, then torch.square) on an fp16 tensor, all 63488 finite inputs,
+    plus the closed forms: negatives and zeros give +0, 3 -> 9, overflow goes to +inf."""
+    from transformers.activations import ACT2FN
+    x = all_finite_fp16()
+    want = ACT2FN["relu2"](torch.from_numpy(x.copy())).numpy()
+    got = O.relu2_fp16(x)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    probe = O.relu2_fp16(np.array([-2.0, -0.0, 0.0, 3.0, 0.5, 300.0], np.float16))
+    assert probe.tolist() == [0.0, 0.0, 0.0, 9.0, 0.25, float("inf")]
+    assert not np.signbit(probe[:3]).any()
+
+
 def test_mlp_gate_up_is_torchs_expression():
     g = torch.randn(64, 96, generator=torch.Generator().manual_seed(0)).half() * 3
     u = torch.randn(64, 96, generator=torch.Generator().manual_seed(1)).half() * 3

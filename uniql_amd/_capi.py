@@ -17,7 +17,7 @@ F_FORCE_SKINNY = 1 << 1
 F_FORCE_TILED = 1 << 2
 F_TRANSPOSE_OUT = 1 << 3
 DT_F16, DT_BF16, DT_F32 = 0, 1, 2
-EPI_NONE, EPI_SILU_MUL = 0, 1
+EPI_NONE, EPI_SILU_MUL, EPI_RELU2 = 0, 1, 2
 
 # every exported symbol with (restype, argtypes); tests check the list against the header
 SIGNATURES = {

@@ -98,7 +98,8 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
     const int rc = check_linear_shape(m, n, k, groups);
     if (rc != UNIQL_OK) return rc;
     const bool transpose = (flags & UNIQL_F_TRANSPOSE_OUT) != 0;
-    if (epilogue != UNIQL_EPI_NONE && epilogue != UNIQL_EPI_SILU_MUL) return UNIQL_E_UNSUPPORTED;
+    if (epilogue != UNIQL_EPI_NONE && epilogue != UNIQL_EPI_SILU_MUL && epilogue != UNIQL_EPI_RELU2)
+        return UNIQL_E_UNSUPPORTED;
     const bool gated = epilogue == UNIQL_EPI_SILU_MUL;
     if (k_in <= 0 || k_in > k || k - k_in >= 128 || (k_in % 8) != 0) return UNIQL_E_SHAPE;
     if (n_out <= 0 || n_out > (gated ? n / 2 : n) || ldd < (transpose ? m : n_out)) return UNIQL_E_SHAPE;
@@ -110,7 +111,7 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
     if (reinterpret_cast<uintptr_t>(D) % (out_f32 ? 4 : 2) != 0) return UNIQL_E_ALIGN;
     if (bias && (reinterpret_cast<uintptr_t>(bias) & 1u)) return UNIQL_E_ALIGN;
     if (residual) {
-        if (gated) return UNIQL_E_UNSUPPORTED;
+        if (epilogue != UNIQL_EPI_NONE) return UNIQL_E_UNSUPPORTED;  // activations feed the next layer, not the residual stream
         if (ldr < n_out) return UNIQL_E_SHAPE;
         if (reinterpret_cast<uintptr_t>(residual) & 1u) return UNIQL_E_ALIGN;
     }
@@ -164,6 +165,7 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
     epi.gated = gated ? 1 : 0;
     epi.out_f32 = out_f32 ? 1 : 0;
     epi.transpose = transpose ? 1 : 0;
+    epi.relu2 = epilogue == UNIQL_EPI_RELU2 ? 1 : 0;
     epi.vec_ok = (!transpose && ldd % 8 == 0 && aligned16(D)) ? 1 : 0;
     if (use_stream)
         return stream_launch(Ain, ld, k_valid, B, S, D, epi, accum, m, n, k, groups, had128, had_scale, tune, st);

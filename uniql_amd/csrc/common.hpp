@@ -97,6 +97,7 @@ struct Epilogue {
     int vec_ok;          // ldd and D allow 16-byte stores of eight fp16 outputs
     int transpose;       // 1: D is [n_store][ldd] with the row index running along the inner axis
                          //    (the reference's output_transpose, "sequence length last")
+    int relu2;           // 1: the stored value is relu(y)^2 of the rounded (and biased) product y
 
     __device__ __forceinline__ size_t offset(int m, int n) const {
         return transpose ? (size_t)n * ldd + m : (size_t)m * ldd + n;
@@ -109,6 +110,10 @@ __device__ __forceinline__ float silu_f32(float x) { return x / (1.0f + expf(-x)
 __device__ __forceinline__ half_t finish_half(const Epilogue& e, int m, int n, float v) {
     half_t y = (half_t)v;
     if (e.bias) y = (half_t)((float)y + (float)e.bias[n]);
+    if (e.relu2) {  // torch.square(relu(y)) on the fp16 tensor: one rounding of the exact square
+        const float r = (float)y > 0.f ? (float)y : 0.f;
+        y = (half_t)(r * r);
+    }
     if (e.residual) y = (half_t)((float)e.residual[(size_t)m * e.ldr + n] + (float)y);
     return y;
 }
@@ -126,6 +131,7 @@ __device__ __forceinline__ void finish_store(const Epilogue& e, void* D, int m, 
     const size_t o = e.offset(m, n);
     if (e.out_f32) {
         if (e.bias) v += (float)e.bias[n];
+        if (e.relu2) v = v > 0.f ? v * v : 0.f;
         if (e.residual) v += (float)e.residual[(size_t)m * e.ldr + n];
         reinterpret_cast<float*>(D)[o] = v;
     } else {

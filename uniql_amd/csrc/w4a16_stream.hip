@@ -414,8 +414,8 @@ static hipError_t launch_waves(const StreamArgs& a, int waves, bool ext, hipStre
 template <bool HAD>
 static hipError_t launch_rows(const StreamArgs& a, int waves, hipStream_t stream) {
     const Epilogue& e = a.epi;
-    const bool ext = e.gated || e.bias || e.residual || e.transpose || e.n_store != a.N || e.ldd != a.N ||
-                     a.k_valid != a.K;
+    const bool ext = e.gated || e.bias || e.residual || e.relu2 || e.transpose || e.n_store != a.N ||
+                     e.ldd != a.N || a.k_valid != a.K;
     if (a.M == 1) return launch_waves<1, HAD>(a, waves, ext, stream);
     if (a.M == 2) return launch_waves<2, HAD>(a, waves, ext, stream);
     if (a.M <= 4) return launch_waves<4, HAD>(a, waves, ext, stream);

@@ -68,13 +68,13 @@ typedef __attribute__((address_space(3))) void* lptr_t;
 __device__ __forceinline__ void store_eight(const Epilogue& e, void* D, int m, int n0, f4 lo, f4 hi) {
     if (e.vec_ok && n0 + 8 <= e.n_store) {
         const size_t o = (size_t)m * e.ldd + n0;
-        if (e.out_f32 && !e.bias && !e.residual) {
+        if (e.out_f32 && !e.bias && !e.residual && !e.relu2) {
             float* d = reinterpret_cast<float*>(D) + o;
             *reinterpret_cast<f4*>(d) = lo;
             *reinterpret_cast<f4*>(d + 4) = hi;
             return;
         }
-        if (!e.out_f32 && !e.bias && !e.residual) {
+        if (!e.out_f32 && !e.bias && !e.residual && !e.relu2) {
             const h2 r0 = h2{(half_t)lo[0], (half_t)lo[1]}, r1 = h2{(half_t)lo[2], (half_t)lo[3]};
             const h2 r2 = h2{(half_t)hi[0], (half_t)hi[1]}, r3 = h2{(half_t)hi[2], (half_t)hi[3]};
             *reinterpret_cast<u32x4*>(reinterpret_cast<half_t*>(D) + o) =
@@ -645,8 +645,8 @@ int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* 
     const int64_t grid = (int64_t)(n / 128) * a.mblocks * a.splits;
     if (grid > 0x7fffffffLL) return UNIQL_E_SHAPE;
     hipError_t e;
-    const bool ext = epi.gated || epi.bias || epi.residual || epi.transpose || epi.n_store != n || epi.ldd != n ||
-                     !epi.vec_ok;
+    const bool ext = epi.gated || epi.bias || epi.residual || epi.relu2 || epi.transpose || epi.n_store != n ||
+                     epi.ldd != n || !epi.vec_ok;
     if (plan.mtiles == 1)
         e = plan.quartets == 2 ? tile_launch_ext<1, 2>(a, ext, (int)grid, stream) : tile_launch_ext<1, 1>(a, ext, (int)grid, stream);
     else if (plan.mtiles == 2)

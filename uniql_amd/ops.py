@@ -140,7 +140,8 @@ def w4a16_gemm_ex(A: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: 
 
 def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: torch.Tensor, size_n: int,
                  size_k: int, *, out_features: int | None = None, bias: torch.Tensor | None = None,
-                 residual: torch.Tensor | None = None, silu_mul: bool = False, had_block: int = 0,
+                 residual: torch.Tensor | None = None, silu_mul: bool = False, relu2: bool = False,
+                 had_block: int = 0,
                  had_scale: float = 1.0, out_f32: bool = False, out: torch.Tensor | None = None,
                  flags: int = 0) -> torch.Tensor:
     """The layer's whole forward in one call (uniql_w4a16_linear): x [m, in_features] with
@@ -149,6 +150,8 @@ def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: t
     layer's `residual + layer(x)`) added with the reference's roundings.  With
     `silu_mul` the packed tensors hold a gate and an up projection interleaved in 64-column
     blocks (layout.interleave_gate_up) and the result is silu(gate) * up, [m, out_features].
+    With `relu2` the result is relu(y)^2 of the (biased) output y, the un-gated MLP front of the
+    squared-ReLU models.
     `out`: optional destination, a 2-D view with unit inner stride (for example a column range
     of a larger buffer)."""
     for t, name in ((x, "x"), (B, "B"), (s, "s"), (workspace, "workspace")):
@@ -166,6 +169,8 @@ def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: t
         raise RuntimeError("B, s and workspace must be contiguous")
     if tuple(B.shape) != (size_k // 16, 2 * size_n) or s.dim() != 2 or s.shape[1] != size_n:
         raise RuntimeError("B / s shapes do not match size_k, size_n")
+    if silu_mul and relu2:
+        raise RuntimeError("silu_mul and relu2 are different epilogues: choose one")
     n_max = size_n // 2 if silu_mul else size_n
     n_out = n_max if out_features is None else int(out_features)
     if not 0 < n_out <= n_max:
@@ -176,8 +181,8 @@ def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: t
             raise RuntimeError("bias must be contiguous float16 with one entry per output column")
     if residual is not None:
         _require_gpu(residual, "residual")
-        if silu_mul:
-            raise RuntimeError("a residual cannot be combined with the gated epilogue")
+        if silu_mul or relu2:
+            raise RuntimeError("a residual cannot be combined with an activation epilogue")
         if residual.dtype != torch.float16 or tuple(residual.shape) != (m, n_out) or residual.stride(1) != 1:
             raise RuntimeError("residual must be float16 [m, out_features] with unit inner stride")
     if k_in % 8 or (m > 1 and x.stride(0) % 8) or x.data_ptr() % 16:
@@ -206,7 +211,8 @@ def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: t
             x.data_ptr(), lda, k_in, B.data_ptr(), s.data_ptr(), bias.data_ptr() if bias is not None else None,
             residual.data_ptr() if residual is not None else None,
             (residual.stride(0) if m > 1 else n_out) if residual is not None else 0,
-            out.data_ptr(), ldd, n_out, _capi.EPI_SILU_MUL if silu_mul else _capi.EPI_NONE,
+            out.data_ptr(), ldd, n_out,
+            _capi.EPI_SILU_MUL if silu_mul else (_capi.EPI_RELU2 if relu2 else _capi.EPI_NONE),
             workspace.data_ptr(), workspace.numel(),
             accum.data_ptr() if accum is not None else None, accum.numel() * 8 if accum is not None else 0,
             temp.data_ptr() if temp is not None else None, need_tmp,

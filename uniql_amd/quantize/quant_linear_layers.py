@@ -95,11 +95,14 @@ class W4A16B16O16Linear(nn.Module):
         return self
 
     @torch.no_grad()
-    def forward(self, x, residual=None):
+    def forward(self, x, residual=None, activation=None):
         """Padding of the input, the product, the cut of the padded output columns and the bias
         (quant_linear_layers.py:92-114) happen inside one kernel call.  Beyond the reference:
         `residual` (same shape as the result) is added in the same call, with the rounding of
-        the decoder layer's `residual + layer(x)`."""
+        the decoder layer's `residual + layer(x)`; `activation="relu2"` applies the squared ReLU
+        of the un-gated MLP (nemotron_h_qblocks.py:588: act_fn(up_proj(x))) to the result."""
+        if activation not in (None, "relu2"):
+            raise ValueError(f"unsupported activation {activation!r} (None or 'relu2')")
         lead = x.shape[:-1]
         x2 = x.reshape(-1, x.shape[-1])
         if x2.stride(-1) != 1:
@@ -107,6 +110,7 @@ class W4A16B16O16Linear(nn.Module):
         y = ops.w4a16_linear(x2, self.weight, self.scale, self.workspace, self.size_n, self.size_k,
                              out_features=self.out_features, bias=None if self.bias is None else self.bias.data,
                              residual=None if residual is None else residual.reshape(-1, self.out_features),
+                             relu2=activation == "relu2",
                              had_block=self.had_block, had_scale=self.had_scale)
         return y.view(*lead, self.out_features)
 
