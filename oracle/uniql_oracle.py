@@ -154,7 +154,7 @@ def fake_quantize_grouped(w: torch.Tensor, group_size: int = GROUP):
     g = w.reshape(-1, group_size, size_n)
     scale = g.abs().max(dim=1, keepdim=True)[0]
     scale *= 2 / 15
-    q = torch.round(g / scale).int()      # NaN (0/0) becomes 0 in .int()
+    q = torch.round(g / scale).int()      # NaN (0/0): INT_MIN on x86 (golden vectors), code 0 after the clamp
     q += 8
     q = torch.clamp(q, 0, 15)
     w_ref = (q - 8) * scale

@@ -96,7 +96,8 @@ def quantize_groupwise(w: torch.Tensor, group_size: int = GROUP_SIZE):
     w: float [K, N].  Returns (w_ref [Kp, N], codes int32 [Kp, N], scale [Kp/g, N])
     with K zero-padded to a multiple of the group.  The arithmetic runs in w's
     dtype with the operation order of quantize_helpers.py:108-118, which is
-    what decides ties and the all-zero-group case (0/0 -> code 8).
+    what decides ties and the all-zero-group case (0/0 = NaN, whose conversion to int32 gives
+    INT_MIN on x86 and so code 0 after the clamp; with scale 0 the weight is -0.0 either way).
     """
     size_k, size_n = w.shape
     pad = (-size_k) % group_size
