@@ -11,6 +11,7 @@ torch.cuda.graph capture.  Errors surface as RuntimeError.
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes
 
 import torch
@@ -24,7 +25,20 @@ __all__ = [
 ]
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_NO_GUARD = contextlib.nullcontext()
+
+
+def _device_guard(device: torch.device):
+    """Makes `device` current for the allocations and the launch; free when it already is."""
+    return _NO_GUARD if torch.cuda.current_device() == device.index else torch.cuda.device(device)
+
+
 def _stream_ptr(device: torch.device) -> int:
+    """The hipStream_t of torch's current stream on `device` (the raw accessor when this torch
+    has it: the public one builds a Stream object on every call)."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -47,7 +61,7 @@ def _capture_id(stream_ptr: int) -> int:
 
 
 def _accumulator(device: torch.device, nbytes: int) -> torch.Tensor:
-    stream = torch.cuda.current_stream(device).cuda_stream
+    stream = _stream_ptr(device)
     key = (device.index, stream)
     buf = _accum_cache.get(key)
     if buf is not None and buf.numel() * 8 >= nbytes:
@@ -115,7 +129,7 @@ def w4a16_gemm_ex(A: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: 
     lib = _capi.load()
     dev = A.device
     out_dtype = torch.float32 if out_f32 else torch.float16
-    with torch.cuda.device(dev):
+    with _device_guard(dev):
         if transpose_out:
             D = torch.zeros((size_n, (size_m + 7) // 8 * 8), dtype=out_dtype, device=dev)
             flags |= _capi.F_TRANSPOSE_OUT
@@ -192,7 +206,7 @@ def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: t
     lib = _capi.load()
     dev = x.device
     out_dtype = torch.float32 if out_f32 else torch.float16
-    with torch.cuda.device(dev):
+    with _device_guard(dev):
         if out is None:
             out = torch.empty((m, n_out), dtype=out_dtype, device=dev)
         elif out.dtype != out_dtype or tuple(out.shape) != (m, n_out) or out.stride(1) != 1 or out.device != dev:
@@ -242,7 +256,7 @@ def w4a16_dequant(B: torch.Tensor, s: torch.Tensor, size_n: int, size_k: int, wa
         raise RuntimeError("B / s shapes do not match size_k, size_n")
     lib = _capi.load()
     dev = B.device
-    with torch.cuda.device(dev):
+    with _device_guard(dev):
         W = torch.empty((size_k, size_n), dtype=torch.float16, device=dev)
         codes = torch.empty((size_k, size_n), dtype=torch.uint8, device=dev) if want_codes else None
         code = lib.uniql_w4a16_dequant(B.data_ptr(), s.data_ptr(), W.data_ptr(),
@@ -270,7 +284,7 @@ def w4a16_quantize(weight: torch.Tensor, given_scale: torch.Tensor | None = None
                 or not given_scale.is_contiguous():
             raise RuntimeError("given_scale must be contiguous float16 [k_pad/128, out_features]")
     lib = _capi.load()
-    with torch.cuda.device(dev):
+    with _device_guard(dev):
         B = torch.empty((k_pad // 16, 2 * n_pad), dtype=torch.int32, device=dev)
         S = torch.empty((k_pad // 128, n_pad), dtype=torch.float16, device=dev)
         code = lib.uniql_w4a16_quantize(weight.data_ptr(), weight.stride(0),
@@ -295,7 +309,7 @@ def w4a16_pack(codes: torch.Tensor, scales: torch.Tensor, pad_out: int = 0):
     n_pad = n + pad_out
     dev = codes.device
     lib = _capi.load()
-    with torch.cuda.device(dev):
+    with _device_guard(dev):
         B = torch.empty((k // 16, 2 * n_pad), dtype=torch.int32, device=dev)
         S = torch.empty((k // 128, n_pad), dtype=torch.float16, device=dev)
         code = lib.uniql_w4a16_pack(codes.data_ptr(), scales.data_ptr(), B.data_ptr(), S.data_ptr(), n, k, n_pad,
@@ -341,7 +355,7 @@ def w4a16_embedding_lookup(input: torch.Tensor, weight: torch.Tensor, scale: tor
     weight_c = weight.detach()
     if not weight_c.is_contiguous() or not scale.is_contiguous():
         raise RuntimeError("weight and scale must be contiguous")
-    with torch.cuda.device(dev):
+    with _device_guard(dev):
         out = torch.empty((*ids.shape, dim), dtype=torch.float16, device=dev)
         code = lib.uniql_w4_embedding_lookup(ids.data_ptr(), ids.numel(), weight_c.data_ptr(), scale.data_ptr(),
                                              out.data_ptr(), vocab, dim, _stream_ptr(dev))
@@ -360,7 +374,7 @@ def w4_embedding_quantize(weight: torch.Tensor):
         raise RuntimeError("embedding_dim and the row stride must be multiples of 8")
     lib = _capi.load()
     dev = weight.device
-    with torch.cuda.device(dev):
+    with _device_guard(dev):
         packed = torch.empty((vocab, dim // 8), dtype=torch.int32, device=dev)
         scales = torch.empty(vocab, dtype=torch.float16, device=dev)
         code = lib.uniql_w4_embedding_quantize(weight.data_ptr(), weight.stride(0) if vocab > 1 else dim,
@@ -404,7 +418,7 @@ def rope_indices_(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torc
         raise RuntimeError("cos, sin and indices must be contiguous")
     lib = _capi.load()
     dev = q.device
-    with torch.cuda.device(dev):
+    with _device_guard(dev):
         code = lib.uniql_rope_indices(q.data_ptr(), q_stride, k.data_ptr(), k_stride, cos.data_ptr(), sin.data_ptr(),
                                       cos.shape[2], indices.data_ptr(), index_bytes, batch * seq, seq, cos.shape[0],
                                       n_qh, n_kh, d, cos.shape[2], _stream_ptr(dev))
@@ -422,7 +436,7 @@ def hadamard_blockwise(x: torch.Tensor, scale: float, block: int | None = None) 
     lib = _capi.load()
     xc = x.contiguous()
     dev = x.device
-    with torch.cuda.device(dev):
+    with _device_guard(dev):
         y = torch.empty_like(xc)
         rows = xc.numel() // dim if dim else 0
         code = lib.uniql_fwht(xc.data_ptr(), y.data_ptr(), rows, dim, block, float(scale),
