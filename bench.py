@@ -201,6 +201,12 @@ def sweep(dev, gen, out_path):
         for name, k, n, hb in PRUNED + MAMBA:
             bench_linear(name, k, (n + 255) // 256 * 256, m, hb, steps=200 if m == 1 else 100)
 
+    # the model's last layer (quantised like the others, quantize_model.py:126-143): one token's
+    # logits stream 4096 x vocabulary weights, more bytes than two decoder layers
+    for name, n in (("lm_head_llama31", 128256), ("lm_head_mamba2", 256000)):
+        for m in (1, 8):
+            bench_linear(name, 4096, n, m, steps=60)
+
     # embedding gather: V = 256000, D = 4096, 2048 ids
     v, d, t = 256000, 4096, 2048
     table = torch.randint(-2 ** 31, 2 ** 31 - 1, (v, d // 8), dtype=torch.int64, device=dev, generator=gen).to(torch.int32)
