@@ -409,3 +409,26 @@ def test_accumulator_cache_across_graphs_and_growth(gpu):
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     ops.reset_accumulators()
+
+
+@pytest.mark.parametrize("m", [1, 5, 40])
+def test_lm_head_shape(gpu, m):
+    """The models' last layer, 4096 -> 128256 (Llama-3.1's vocabulary; quantised like the other
+    layers, quantize_model.py:126-143): 1002 column strips in one launch.  Too large for the CPU
+    oracle in a test's time: the reference product is torch's fp32 matmul on the GPU with the
+    weights from uniql_w4a16_dequant, which the tests above hold bit-exact against the oracle."""
+    from uniql_amd import ops
+    k, n = 4096, 128256
+    g = torch.Generator(device=gpu).manual_seed(77 + m)
+    b = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 16, 2 * n), generator=g, device=gpu, dtype=torch.int64).to(torch.int32)
+    s = (torch.rand(k // 128, n, generator=g, device=gpu) * 0.016 + 0.004).half()
+    x = torch.randn(m, k, generator=g, device=gpu).half()
+    ws = workspace_for(n, gpu)
+    w = ops.w4a16_dequant(b, s, n, k)
+    ref = (x.float() @ w.float()).cpu().numpy()
+    del w
+    y32 = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k, out_f32=True).cpu().numpy()
+    assert np.abs(y32 - ref).max() < (1e-4 * np.sqrt(k) + 2e-4 if m <= 16 else 5e-4)
+    y = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k)
+    assert np.array_equal(y.cpu().numpy(), y32.astype(np.float16))
+    check_layer_output(y.cpu().numpy(), ref)
