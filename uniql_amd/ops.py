@@ -51,6 +51,8 @@ _accum_cache: dict = {}
 _accum_retired: list = []
 # Buffers born inside a graph capture, keyed by the capture as well: their zero fill is a node
 # of that graph, so they are only known to be zero when that graph replays and serve nothing else.
+# They are kept until reset_accumulators() (one buffer per capture that needed one; a capture on
+# a stream that already ran an eager call uses that stream's eager buffer instead).
 _accum_in_capture: dict = {}
 
 
