@@ -144,6 +144,16 @@ enum { UNIQL_EPI_NONE = 0, UNIQL_EPI_SILU_MUL = 1, UNIQL_EPI_RELU2 = 2 };
 
 size_t uniql_w4a16_linear_temp_bytes(int m, int n, int k, int k_in, int had_block);
 
+/* Sizes of `accum` and `temp` for one call with these flags (the two functions above and
+ * uniql_w4a16_gemm_accum_bytes answer for flags = 0; forced kernels or tuning fields can need
+ * more).  `temp` holds the rotated or zero-padded copy of the activations and, when the tiled
+ * kernel splits K over workgroups, one fp32 partial tile per (output tile, split); `accum` then
+ * holds one arrival count per output tile.  No counterpart in the reference, whose wrapper
+ * allocates its reduction buffer itself (csrc/linear/marlin_gemm_kernel.cuh:1018). */
+int uniql_w4a16_linear_workspace(int m, int n, int k, int k_in, int had_block, unsigned flags,
+                                 size_t* accum_bytes, size_t* temp_bytes);
+
+
 int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, const void* S, const void* bias,
                        const void* residual, int64_t ldr,
                        void* D, int64_t ldd, int n_out, int epilogue,

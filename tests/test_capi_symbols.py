@@ -39,14 +39,30 @@ def test_host_only_entry_points(lib):
     assert lib.uniql_abi_version() == 1
     assert lib.uniql_status_string(0) == b"ok"
     assert b"NULL" in lib.uniql_status_string(-1)
-    # one 64-bit word per output element of a (<= 64 row) slab when K can be split
+    # streaming kernel: one 64-bit word per output element of a (<= 16 row) slab when K can be
+    # split; tiled kernel: one word per output tile (far fewer); the answer covers both
     assert lib.uniql_w4a16_gemm_accum_bytes(1, 4096, 4096) == 4096 * 8
-    assert lib.uniql_w4a16_gemm_accum_bytes(100, 4096, 4096) == 100 * 4096 * 8
+    assert lib.uniql_w4a16_gemm_accum_bytes(100, 4096, 4096) == 16 * 4096 * 8
     assert lib.uniql_w4a16_gemm_accum_bytes(4096, 4096, 4096) == 16 * 4096 * 8
     assert lib.uniql_w4a16_gemm_accum_bytes(1, 4096, 512) == 0
     assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 8192) == 2 * 8192 * 2
     assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 128) == 2 * 8192 * 2
     assert lib.uniql_w4a16_gemm_temp_bytes(2, 4096, 8192, 0) == 0
+    import ctypes
+    acc, tmp = ctypes.c_size_t(7), ctypes.c_size_t(7)
+    ws = lib.uniql_w4a16_linear_workspace
+    assert ws(1, 4096, 4096, 4096, 0, 0, ctypes.byref(acc), ctypes.byref(tmp)) == 0
+    assert (acc.value, tmp.value) == (4096 * 8, 0)                      # streaming kernel, K split with atomics
+    assert ws(1024, 4096, 4096, 4096, 0, 0, ctypes.byref(acc), ctypes.byref(tmp)) == 0
+    assert (acc.value, tmp.value) == (0, 0)                             # tiled kernel, whole K per workgroup
+    # tiled kernel forced to split K four ways with 128-row tiles: a count per tile, a partial tile per split
+    forced = (4 << 8) | (4 << 16)
+    assert ws(256, 4096, 4096, 4096, 0, forced, ctypes.byref(acc), ctypes.byref(tmp)) == 0
+    assert (acc.value, tmp.value) == (32 * 2 * 8, 4 * 256 * 4096 * 4)
+    assert ws(256, 4096, 4096, 4000, 0, forced, ctypes.byref(acc), ctypes.byref(tmp)) == 0
+    assert tmp.value == 256 * 4096 * 2 + 4 * 256 * 4096 * 4             # + the zero-padded copy of the input
+    assert ws(1, 4096 + 64, 4096, 4096, 0, 0, ctypes.byref(acc), ctypes.byref(tmp)) == -2
+    assert ws(1, 4096, 4096, 4096, 0, 0, None, ctypes.byref(tmp)) == -1
     assert lib.uniql_stream_capture_id(None, None) == -1    # the result pointer is checked before any HIP call
 
 

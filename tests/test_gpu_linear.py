@@ -134,6 +134,30 @@ def test_tile_kernel_k_splits(gpu, splits):
     assert np.array_equal(y32, again)                          # integer accumulation: order-independent
 
 
+@pytest.mark.parametrize("m,k,n,splits,mt", [(300, 1536, 1280, 3, 0), (200, 1024, 896, 4, 1), (257, 1536, 768, 3, 2),
+                                             (300, 2048, 640, 4, 4)])
+def test_tile_split_exchange_is_ordered(gpu, m, k, n, splits, mt):
+    """K split over workgroups of the tiled kernel: partial tiles go through scratch memory and
+    the last workgroup of a tile adds them.  The result must not depend on which workgroup that
+    is, nor may it ever read a slot before it is complete: the same call many times over, with
+    the scratch area dirtied in between, gives the same bits every time and the right values."""
+    from uniql_amd import ops
+    p = make_linear_problem(m, k, n, seed=m + k + n)
+    x, b, s = to_gpu(p, gpu)
+    ws = workspace_for(n, gpu)
+    flags = F_FORCE_TILED | (splits << 8) | (mt << 16)
+    first = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k, out_f32=True, flags=flags)
+    assert np.abs(first.cpu().numpy() - reference_product(p, exact=True)).max() < 3e-4
+    same = torch.ones((), dtype=torch.bool, device=gpu)
+    for rep in range(1000):
+        if rep % 10 == 0:   # dirty what the allocator hands out next as scratch area
+            junk = torch.full((splits * m * n + 4096,), float("nan"), dtype=torch.float32, device=gpu)
+            del junk
+        again = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k, out_f32=True, flags=flags)
+        same &= (first == again).all()
+    assert bool(same)
+
+
 @pytest.mark.parametrize("mt", [1, 2])
 @pytest.mark.parametrize("m,k,n", [(32, 256, 128), (100, 1024, 256), (256, 4096, 512), (64, 768, 128), (33, 640, 256)])
 def test_tile_kernel_two_wave_quartets(gpu, m, k, n, mt):
@@ -350,7 +374,7 @@ def test_accumulator_cache_across_graphs_and_growth(gpu):
     ops.reset_accumulators()
     small = make_linear_problem(1, 4096, 512, seed=311)       # K split with atomics, small accumulator
     other = make_linear_problem(2, 2048, 256, seed=312)
-    large = make_linear_problem(48, 4096, 2048, seed=313)     # tiled kernel with K splits: more words
+    large = make_linear_problem(16, 1024, 8192, seed=313)     # 16 x 8192 words: beyond the cache's first size
     xs, bs, ss = to_gpu(small, gpu)
     xo, bo, so = to_gpu(other, gpu)
     xl, bl, sl = to_gpu(large, gpu)
@@ -363,7 +387,7 @@ def test_accumulator_cache_across_graphs_and_growth(gpu):
         return ops.w4a16_gemm_ex(xo, bo, so, ws_o, 2, 256, 2048)
 
     def run_large():
-        return ops.w4a16_gemm_ex(xl, bl, sl, ws_l, 48, 2048, 4096)
+        return ops.w4a16_gemm_ex(xl, bl, sl, ws_l, 16, 8192, 1024)
 
     # first use of the capture stream happens inside the captures
     g1, g2 = torch.cuda.CUDAGraph(), torch.cuda.CUDAGraph()

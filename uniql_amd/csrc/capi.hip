@@ -8,7 +8,9 @@ int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const 
                   unsigned tune, hipStream_t stream);
 size_t stream_accum_bytes(int m, int n, int k);
 int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, const Epilogue& epi, void* accum,
-                size_t accum_bytes, int m, int n, int k, int groups, unsigned tune, hipStream_t stream);
+                size_t accum_bytes, void* part, size_t part_bytes, int m, int n, int k, int groups, unsigned tune,
+                hipStream_t stream);
+size_t tile_part_bytes(int m, int n, int k, unsigned tune);
 int pad_rows_launch(const void* A, int64_t lda, int k_in, void* dst, int k, int m, hipStream_t stream);
 size_t tile_accum_bytes(int m, int n, int k, unsigned tune = 0);
 int dequant_launch(const void* B, const void* S, void* W, uint8_t* codes, int n, int k, int groups,
@@ -71,19 +73,53 @@ const char* uniql_status_string(int code) {
 // rows up to this many take the weight-streaming kernel, more take the tiled one
 static constexpr int kStreamMaxM = 16;
 
+// which kernel takes a call
+static bool takes_stream_kernel(int m, unsigned flags) {
+    bool use_stream = m <= kStreamMaxM;
+    if (flags & UNIQL_F_FORCE_SKINNY) use_stream = true;
+    if (flags & UNIQL_F_FORCE_TILED) use_stream = false;
+    return use_stream;
+}
+
+// bytes of the rotated or zero-padded copy of the activations at the start of `temp`: every
+// rotation except the 128-block one fused into the streaming kernel, and padding whenever the
+// kernel cannot guard its own loads (tiled kernel) or a rotation comes first
+static size_t activation_copy_bytes(int m, int k, int k_in, int had_block, bool use_stream) {
+    const bool rotate_first = had_block != 0 && !(had_block == 128 && use_stream);
+    const bool pad_first = k_in != k && (rotate_first || !use_stream);
+    return (rotate_first || pad_first) ? round256((size_t)m * k * sizeof(half_t)) : 0;
+}
+
+int uniql_w4a16_linear_workspace(int m, int n, int k, int k_in, int had_block, unsigned flags, size_t* accum_bytes,
+                                 size_t* temp_bytes) {
+    if (!accum_bytes || !temp_bytes) return UNIQL_E_NULL;
+    *accum_bytes = *temp_bytes = 0;
+    if (m < 0 || n <= 0 || k <= 0 || n % 128 != 0 || k % 128 != 0) return UNIQL_E_SHAPE;
+    if (m == 0) return UNIQL_OK;
+    const bool use_stream = takes_stream_kernel(m, flags);
+    const unsigned tune = flags >> 8;
+    *accum_bytes = round256(use_stream ? stream_accum_bytes(m, n, k) : tile_accum_bytes(m, n, k, tune));
+    // a strided input ahead of a separate rotation is compacted into the copy as well: count it
+    const size_t act = had_block != 0 && !(had_block == 128 && use_stream)
+                           ? round256((size_t)m * k * sizeof(half_t))
+                           : activation_copy_bytes(m, k, k_in, had_block, use_stream);
+    *temp_bytes = act + (use_stream ? 0 : round256(tile_part_bytes(m, n, k, tune)));
+    return UNIQL_OK;
+}
+
 size_t uniql_w4a16_gemm_accum_bytes(int m, int n, int k) {
     if (m <= 0 || n <= 0 || k <= 0 || n % 128 != 0 || k % 128 != 0) return 0;
-    // enough for either kernel, so that the forcing flags never need a bigger buffer
+    // enough for either kernel with its own plan (forced tuning fields: uniql_w4a16_linear_workspace)
     const size_t a = stream_accum_bytes(m, n, k), b = tile_accum_bytes(m, n, k);
     return round256(a > b ? a : b);
 }
 
 size_t uniql_w4a16_linear_temp_bytes(int m, int n, int k, int k_in, int had_block) {
-    if (m <= 0 || n <= 0 || k <= 0) return 0;
-    // a rotated (every block width except the 128 fused into the streaming kernel, and 128 too
-    // once the tiled kernel may take the call) or zero-padded copy of the activations
-    if (had_block != 0 || k_in != k) return round256((size_t)m * k * sizeof(half_t));
-    return 0;
+    if (m <= 0 || n <= 0 || k <= 0 || n % 128 != 0 || k % 128 != 0) return 0;
+    // the copy of the activations (as if the tiled kernel took the call: the larger case) and the
+    // partial tiles of the tiled kernel's own plan
+    const size_t act = (had_block != 0 || k_in != k) ? round256((size_t)m * k * sizeof(half_t)) : 0;
+    return act + (takes_stream_kernel(m, 0) ? 0 : round256(tile_part_bytes(m, n, k, 0)));
 }
 
 size_t uniql_w4a16_gemm_temp_bytes(int m, int n, int k, int had_block) {
@@ -118,14 +154,12 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
     if (workspace && workspace_len < n / 128) return UNIQL_E_WORKSPACE;
     if (had_block != 0 && (!is_pow2(had_block) || had_block < 2 || had_block > 32768 || k % had_block != 0))
         return UNIQL_E_SHAPE;
-    const size_t need_accum = uniql_w4a16_gemm_accum_bytes(m, n, k);
-    if (need_accum > 0 && (!accum || accum_bytes < need_accum)) return UNIQL_E_WORKSPACE;
     if ((accum && !aligned16(accum)) || (temp && !aligned16(temp))) return UNIQL_E_ALIGN;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-
-    bool use_stream = m <= kStreamMaxM;
-    if (flags & UNIQL_F_FORCE_SKINNY) use_stream = true;
-    if (flags & UNIQL_F_FORCE_TILED) use_stream = false;
+    const bool use_stream = takes_stream_kernel(m, flags);
+    const unsigned tune = flags >> 8;  // tuning fields, see the header
+    const size_t need_accum = round256(use_stream ? stream_accum_bytes(m, n, k) : tile_accum_bytes(m, n, k, tune));
+    if (need_accum > 0 && (!accum || accum_bytes < need_accum)) return UNIQL_E_WORKSPACE;
 
     const void* Ain = A;
     int64_t ld = lda;
@@ -135,14 +169,11 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
     // the transform kernel reads dense rows of k values: a strided or short input is first copied
     // (and zero-padded) into the temporary buffer, then rotated there in place
     const bool pad_first = rotate_first ? (k_in != k || lda != k) : (k_in != k && !use_stream);
-    if (rotate_first || pad_first) {
-        if (!temp || temp_bytes < round256((size_t)m * k * sizeof(half_t))) return UNIQL_E_WORKSPACE;
-    }
-    const unsigned tune = flags >> 8;  // tuning fields, see the header
-    if (!use_stream) {  // a forced number of K splits may need more words than the default plan
-        const size_t need = tile_accum_bytes(m, n, k, tune);
-        if (need > 0 && (!accum || accum_bytes < need)) return UNIQL_E_WORKSPACE;
-    }
+    // temp: the copy of the activations, then the tiled kernel's partial tiles when it splits K
+    const size_t act_bytes = (rotate_first || pad_first) ? round256((size_t)m * k * sizeof(half_t)) : 0;
+    const size_t part_bytes = use_stream ? 0 : tile_part_bytes(m, n, k, tune);
+    if (act_bytes + part_bytes > 0 && (!temp || temp_bytes < act_bytes + part_bytes)) return UNIQL_E_WORKSPACE;
+    void* part = part_bytes ? reinterpret_cast<char*>(temp) + act_bytes : nullptr;
     if (pad_first) {
         const int e = pad_rows_launch(A, lda, k_in, temp, k, m, st);
         if (e != UNIQL_OK) return e;
@@ -169,7 +200,7 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
     epi.vec_ok = (!transpose && ldd % 8 == 0 && aligned16(D)) ? 1 : 0;
     if (use_stream)
         return stream_launch(Ain, ld, k_valid, B, S, D, epi, accum, m, n, k, groups, had128, had_scale, tune, st);
-    return tile_launch(Ain, ld, B, S, D, epi, accum, accum_bytes, m, n, k, groups, tune, st);
+    return tile_launch(Ain, ld, B, S, D, epi, accum, accum_bytes, part, part_bytes, m, n, k, groups, tune, st);
 }
 
 int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, void* D, const int32_t* workspace,

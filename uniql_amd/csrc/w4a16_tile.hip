@@ -46,7 +46,8 @@ struct TileArgs {
     const half_t* S;
     const half_t* X;
     void* D;
-    unsigned long long* accum;  // [M][N] sum|count words (splits > 1), zero on entry and exit
+    unsigned long long* accum;  // one arrival count per output tile (splits > 1), zero on entry and exit
+    float* part;                // [tile][split][32 MT][128] partial tiles (splits > 1), any contents
     int64_t ldx;
     int M, N, K;
     int G;            // K / 128
@@ -116,6 +117,34 @@ __device__ __forceinline__ void store_eight_gated(const Epilogue& e, void* D, in
         finish_store_gated(e, D, m, n0 + i, glo[i], ulo[i]);
         finish_store_gated(e, D, m, n0 + 4 + i, ghi[i], uhi[i]);
     }
+}
+
+// Eight fp32 partial sums to / from a workgroup's slot of the split-K scratch area: relaxed
+// device-scope accesses (write-through stores, loads that do not trust a stale cache line), so
+// workgroups on different XCDs exchange them without flushing or invalidating a whole L2.  The
+// four 8-byte words of a unit lie `stride` words apart: word i of all threads of the workgroup is
+// one contiguous run, so every store instruction writes whole cache lines.
+__device__ __forceinline__ unsigned long long pack_floats(float a, float b) {
+    return (unsigned long long)__float_as_uint(a) | ((unsigned long long)__float_as_uint(b) << 32);
+}
+__device__ __forceinline__ void store_partial(unsigned long long* d, int stride, f4 lo, f4 hi) {
+    __hip_atomic_store(d, pack_floats(lo[0], lo[1]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(d + stride, pack_floats(lo[2], lo[3]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(d + 2 * stride, pack_floats(hi[0], hi[1]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(d + 3 * stride, pack_floats(hi[2], hi[3]), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void add_partial(const unsigned long long* p, int stride, f4& lo, f4& hi) {
+    unsigned long long w[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) w[i] = __hip_atomic_load(p + i * stride, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    lo[0] += __uint_as_float((uint32_t)w[0]);
+    lo[1] += __uint_as_float((uint32_t)(w[0] >> 32));
+    lo[2] += __uint_as_float((uint32_t)w[1]);
+    lo[3] += __uint_as_float((uint32_t)(w[1] >> 32));
+    hi[0] += __uint_as_float((uint32_t)w[2]);
+    hi[1] += __uint_as_float((uint32_t)(w[2] >> 32));
+    hi[2] += __uint_as_float((uint32_t)w[3]);
+    hi[3] += __uint_as_float((uint32_t)(w[3] >> 32));
 }
 
 template <int MT, int KW = 1>
@@ -420,6 +449,38 @@ __global__ __launch_bounds__(256 * KW, 1) void w4a16_tile_kernel(const TileArgs 
     constexpr int NW = 4 * KW;
     const bool split_k = a.splits > 1;
     const bool gated = EXT && a.epi.gated != 0;  // uniform
+
+    // one finished unit: eight consecutive columns c0.. of output row m
+    auto emit = [&](int m, int c0, f4 lo, f4 hi) {
+        if constexpr (EXT) {
+            store_eight(a.epi, a.D, m, 128 * strip + c0, lo, hi);
+        } else {
+            const size_t o = (size_t)m * a.N + 128 * strip + c0;
+            if (a.epi.out_f32) {
+                float* d = reinterpret_cast<float*>(a.D) + o;
+                *reinterpret_cast<f4*>(d) = lo;
+                *reinterpret_cast<f4*>(d + 4) = hi;
+            } else {
+                const h2 r0 = h2{(half_t)lo[0], (half_t)lo[1]}, r1 = h2{(half_t)lo[2], (half_t)lo[3]};
+                const h2 r2 = h2{(half_t)hi[0], (half_t)hi[1]}, r3 = h2{(half_t)hi[2], (half_t)hi[3]};
+                *reinterpret_cast<u32x4*>(reinterpret_cast<half_t*>(a.D) + o) =
+                    u32x4{h2_to_bits(r0), h2_to_bits(r1), h2_to_bits(r2), h2_to_bits(r3)};
+            }
+        }
+    };
+
+    // K split over workgroups: every workgroup writes its 32 MT x 128 partial tile (fp32) to its
+    // slot of the scratch area, then counts itself in the tile's word; whoever completes the count
+    // adds the slots in split order (so the sum does not depend on who came last) and stores.
+    // A slot holds the tile as 512 MT units of (row, 8 columns); unit u of M tile mt (row u / 16,
+    // columns 8 (u % 16)..) is the four words ((mt UPT + u / T) 4 + i) T + u % T, i = 0..3, with
+    // T the workgroup's thread count: the thread that reduces a unit writes it, lane after lane.
+    const int tile = mblock * nstrips + strip;
+    constexpr int T = 256 * KW, UPT = 512 / T, kSlotWords = ROWS * 64;
+    unsigned long long* part_tile =
+        split_k ? reinterpret_cast<unsigned long long*>(a.part) + (size_t)tile * a.splits * kSlotWords : nullptr;
+    unsigned long long* part_mine = split_k ? part_tile + (size_t)split * kSlotWords : nullptr;
+    auto unit_word = [&](int mt, int unit) { return ((mt * UPT + unit / T) * 4) * T + unit % T; };
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
         if (m0 + mt * 32 < a.M) {  // uniform
@@ -434,91 +495,77 @@ __global__ __launch_bounds__(256 * KW, 1) void w4a16_tile_kernel(const TileArgs 
                             f4{acc[mt][op][4 * j4], acc[mt][op][4 * j4 + 1], acc[mt][op][4 * j4 + 2], acc[mt][op][4 * j4 + 3]};
             }
             __syncthreads();
-            if (!split_k) {
-                // gated: the 32 x 64 output block is 256 units, one per thread (columns c0 and
-                // c0 + 64 of the strip); else 512 units, two per thread
-                const int units = gated ? 256 : 512;
-                for (int unit = tid; unit < units; unit += 256 * KW) {
-                    const int row = gated ? unit >> 3 : unit >> 4;
-                    const int c0 = gated ? (unit & 7) * 8 : (unit & 15) * 8;
-                    const int m = m0 + mt * 32 + row;
-                    const float* src = red + row * kRedStride + c0;
-                    f4 lo = *reinterpret_cast<const f4*>(src), hi = *reinterpret_cast<const f4*>(src + 4);
+            // gated and not split: the 32 x 64 output block is 256 units, one per thread (columns
+            // c0 and c0 + 64 of the strip); else 512 units, two per thread
+            const bool pairs_now = gated && !split_k;
+            const int units = pairs_now ? 256 : 512;
+            for (int unit = tid; unit < units; unit += 256 * KW) {
+                const int row = pairs_now ? unit >> 3 : unit >> 4;
+                const int c0 = pairs_now ? (unit & 7) * 8 : (unit & 15) * 8;
+                const int m = m0 + mt * 32 + row;
+                const float* src = red + row * kRedStride + c0;
+                f4 lo = *reinterpret_cast<const f4*>(src), hi = *reinterpret_cast<const f4*>(src + 4);
+#pragma unroll
+                for (int ww = 1; ww < NW; ++ww) {
+                    lo += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride);
+                    hi += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride + 4);
+                }
+                if (split_k) {
+                    if (m < a.M) store_partial(part_mine + unit_word(mt, unit), T, lo, hi);  // rows that exist only
+                } else if (!gated) {
+                    if (m < a.M) emit(m, c0, lo, hi);
+                } else {
+                    f4 ulo = *reinterpret_cast<const f4*>(src + 64), uhi = *reinterpret_cast<const f4*>(src + 68);
 #pragma unroll
                     for (int ww = 1; ww < NW; ++ww) {
-                        lo += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride);
-                        hi += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride + 4);
+                        ulo += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride + 64);
+                        uhi += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride + 68);
                     }
-                    if (!gated) {
-                        if (m < a.M) {
-                            if constexpr (EXT) {
-                                store_eight(a.epi, a.D, m, 128 * strip + c0, lo, hi);
-                            } else {
-                                const size_t o = (size_t)m * a.N + 128 * strip + c0;
-                                if (a.epi.out_f32) {
-                                    float* d = reinterpret_cast<float*>(a.D) + o;
-                                    *reinterpret_cast<f4*>(d) = lo;
-                                    *reinterpret_cast<f4*>(d + 4) = hi;
-                                } else {
-                                    const h2 r0 = h2{(half_t)lo[0], (half_t)lo[1]}, r1 = h2{(half_t)lo[2], (half_t)lo[3]};
-                                    const h2 r2 = h2{(half_t)hi[0], (half_t)hi[1]}, r3 = h2{(half_t)hi[2], (half_t)hi[3]};
-                                    *reinterpret_cast<u32x4*>(reinterpret_cast<half_t*>(a.D) + o) =
-                                        u32x4{h2_to_bits(r0), h2_to_bits(r1), h2_to_bits(r2), h2_to_bits(r3)};
-                                }
-                            }
-                        }
-                    } else {
-                        f4 ulo = *reinterpret_cast<const f4*>(src + 64), uhi = *reinterpret_cast<const f4*>(src + 68);
-#pragma unroll
-                        for (int ww = 1; ww < NW; ++ww) {
-                            ulo += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride + 64);
-                            uhi += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride + 68);
-                        }
-                        if (m < a.M) store_eight_gated(a.epi, a.D, m, 64 * strip + c0, lo, hi, ulo, uhi);
-                    }
-                }
-            } else {
-                // K is also split over workgroups: one atomic per element, neighbouring lanes on
-                // neighbouring words (a wave touches 512 contiguous bytes per instruction)
-                const int col_out = tid & 127;
-                for (int i = 0; i < 16 / KW; ++i) {
-                    const int row = (tid >> 7) + 2 * KW * i;
-                    const int m = m0 + mt * 32 + row;
-                    if (m >= a.M) continue;
-                    const float* src = red + row * kRedStride + col_out;
-                    float sum = (src[0] + src[32 * kRedStride]) + (src[64 * kRedStride] + src[96 * kRedStride]);
-                    if (KW == 2)
-                        sum += (src[128 * kRedStride] + src[160 * kRedStride]) + (src[192 * kRedStride] + src[224 * kRedStride]);
-                    const int n_out = 128 * strip + col_out;
-                    unsigned long long* word = a.accum + (size_t)m * a.N + n_out;
-                    if (!gated) {
-                        float total;
-                        if (accum_add(word, sum, a.splits, total)) {
-                            if constexpr (EXT) {
-                                finish_store(a.epi, a.D, m, n_out, total);
-                            } else if (a.epi.out_f32) {
-                                reinterpret_cast<float*>(a.D)[(size_t)m * a.N + n_out] = total;
-                            } else {
-                                reinterpret_cast<half_t*>(a.D)[(size_t)m * a.N + n_out] = (half_t)total;
-                            }
-                            accum_reset(word);
-                        }
-                    } else if (col_out < 64) {
-                        const float* usrc = src + 64;
-                        float usum = (usrc[0] + usrc[32 * kRedStride]) + (usrc[64 * kRedStride] + usrc[96 * kRedStride]);
-                        if (KW == 2)
-                            usum += (usrc[128 * kRedStride] + usrc[160 * kRedStride]) +
-                                    (usrc[192 * kRedStride] + usrc[224 * kRedStride]);
-                        float total_g, total_u;
-                        if (accum_add_pair(word, word + 64, sum, usum, a.splits, total_g, total_u)) {
-                            finish_store_gated(a.epi, a.D, m, 64 * strip + col_out, total_g, total_u);
-                            accum_reset(word);
-                        }
-                    }
+                    if (m < a.M) store_eight_gated(a.epi, a.D, m, 64 * strip + c0, lo, hi, ulo, uhi);
                 }
             }
         }
     }
+    if (!split_k) return;  // uniform
+
+    // Every thread waits for its own partial stores (device-scope write-through stores) to be
+    // acknowledged before the barrier - the barrier alone does not wait for outstanding stores -
+    // so the slot is in place before thread 0 counts the workgroup in; the last workgroup reads
+    // the slots with device-scope loads.  No cache-wide write-back or invalidate is involved.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    int* last_flag = reinterpret_cast<int*>(lds_all);
+    if (tid == 0) {
+        const unsigned long long old =
+            __hip_atomic_fetch_add(a.accum + tile, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *last_flag = (int)old == a.splits - 1;
+    }
+    __syncthreads();
+    if (*last_flag == 0) return;  // uniform
+    const int units = gated ? 256 : 512;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+        if (m0 + mt * 32 >= a.M) break;  // uniform
+        for (int unit = tid; unit < units; unit += 256 * KW) {
+            const int row = gated ? unit >> 3 : unit >> 4;
+            const int c0 = gated ? (unit & 7) * 8 : (unit & 15) * 8;
+            const int m = m0 + mt * 32 + row;
+            if (m >= a.M) continue;
+            // the unit's number in the writers' enumeration (16 units per row); a gated pair's up
+            // half is 8 units on
+            const int wunit = row * 16 + (c0 >> 3);
+            const unsigned long long* src = part_tile + unit_word(mt, wunit);
+            const unsigned long long* usrc = part_tile + unit_word(mt, wunit + 8);
+            f4 lo = f4{0.f, 0.f, 0.f, 0.f}, hi = lo, ulo = lo, uhi = lo;
+            for (int sp = 0; sp < a.splits; ++sp) {
+                add_partial(src + (size_t)sp * kSlotWords, T, lo, hi);
+                if (gated) add_partial(usrc + (size_t)sp * kSlotWords, T, ulo, uhi);
+            }
+            if (!gated) emit(m, c0, lo, hi);
+            else store_eight_gated(a.epi, a.D, m, 64 * strip + c0, lo, hi, ulo, uhi);
+        }
+    }
+    if (tid == 0) __hip_atomic_store(a.accum + tile, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // ---------------------------------------------------------------------------------
@@ -530,11 +577,23 @@ struct TilePlan {
 };
 static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_override = 0, int kw_override = 0);
 
-// tune: the same fields as tile_launch takes
+static TilePlan tile_plan_tuned(int m, int n, int k, unsigned tune) {
+    return tile_plan(m, n, k, (int)(tune & 0xffu), (int)((tune >> 8) & 0xfu), (int)((tune >> 12) & 0x3u));
+}
+
+// What a plan that splits K over workgroups needs (tune: the same fields as tile_launch takes):
+// one arrival count per output tile in `accum` (zero on entry, zero again on exit) and one fp32
+// partial tile per (tile, split) in a scratch area whose contents do not matter.
 size_t tile_accum_bytes(int m, int n, int k, unsigned tune) {
-    // one word per output element, only when the plan splits K over workgroups
-    const TilePlan plan = tile_plan(m, n, k, (int)(tune & 0xffu), (int)((tune >> 8) & 0xfu), (int)((tune >> 12) & 0x3u));
-    return plan.splits > 1 ? (size_t)m * n * sizeof(unsigned long long) : 0;
+    const TilePlan plan = tile_plan_tuned(m, n, k, tune);
+    if (plan.splits <= 1) return 0;
+    return (size_t)(n / 128) * ceil_div_i(m, 32 * plan.mtiles) * sizeof(unsigned long long);
+}
+size_t tile_part_bytes(int m, int n, int k, unsigned tune) {
+    const TilePlan plan = tile_plan_tuned(m, n, k, tune);
+    if (plan.splits <= 1) return 0;
+    const size_t tiles = (size_t)(n / 128) * ceil_div_i(m, 32 * plan.mtiles);
+    return tiles * plan.splits * (32 * plan.mtiles * 128) * sizeof(float);
 }
 
 // Measured on MI355X, in units of the time one MT = 4 workgroup takes for its K loop when every
@@ -546,10 +605,10 @@ size_t tile_accum_bytes(int m, int n, int k, unsigned tune) {
 //     512, 1.62 per started round of 1024;
 //   * a grid that gives a compute unit at most one MT = 1 or MT = 2 workgroup runs faster with two
 //     wave quartets per workgroup (factors 0.85 and 0.92);
-//   * the exchange of partial sums costs one 64-bit atomic per output element and K split,
-//     about 150 G atomics/s for the chip.
-// So: the MT with the cheapest grid; K splits only for MT = 1 grids that cannot fill the chip,
-// and only while the atomics cost less than the K loop they save; two quartets whenever the final
+//   * K split over workgroups: every workgroup writes its fp32 partial tile to scratch memory and
+//     the last one to arrive adds them (about 1 to 1.5 us per MB of partial tiles).
+// So: the MT with the cheapest grid; K splits while the grid stays within one workgroup per compute
+// unit and the partial tiles stay small against the weights; two quartets whenever the final
 // grid has at most 256 workgroups of MT <= 2 and every workgroup gets an even number of groups.
 static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_override, int kw_override) {
     TilePlan p;
@@ -567,21 +626,19 @@ static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_overr
     if (cost2 < cost4 && cost2 <= cost1) p.mtiles = 2;
     else if (cost1 < cost4) p.mtiles = 1;
     if (m <= 32) p.mtiles = 1;
+    // a long K loop over few 64-row tiles: two K splits of 64-row tiles beat 32-row tiles (every
+    // weight is expanded for twice the rows; down_proj at M = 256: 545 -> 650 TFLOP/s)
+    if (p.mtiles == 1 && G >= 64 && m >= 64 && t2 <= 128) p.mtiles = 2;
     if (mt_override == 1 || mt_override == 2 || mt_override == 4) p.mtiles = mt_override;
     const int64_t tiles = (int64_t)strips * ceil_div_i(m, 32 * p.mtiles);
     int splits = 1;
     if (splits_override > 0) {
         splits = splits_override;
-    } else if (p.mtiles == 1 && tiles < 256) {
-        double best = G * 0.7;
-        for (int sp = 2; sp <= 16; sp *= 2) {
-            if (G / sp < 4 || tiles * sp > 1024) break;
-            const double cost = (double)ceil_div_i(G, sp) * 0.7 + (double)m * n * sp / 150e3 + 5.0;
-            if (cost < best) {
-                best = cost;
-                splits = sp;
-            }
-        }
+    } else {
+        // K splits while the grid stays within one workgroup per compute unit, every workgroup
+        // keeps at least 8 groups, and the partial tiles (m x n x 4 bytes per split, written and
+        // read once) stay below a quarter of the packed weights the launch streams
+        while (tiles * (2 * splits) <= 256 && G / (2 * splits) >= 8 && (int64_t)(2 * splits) * m * 16 <= k) splits *= 2;
     }
     if (splits > G) splits = G;
     if (splits > 255) splits = 255;
@@ -622,11 +679,14 @@ static hipError_t tile_launch_ext(const TileArgs& a, bool ext, int grid, hipStre
 // tune: bits 0..7 force the number of K splits, bits 8..11 the number of 32-row M tiles per
 // workgroup, bits 12..13 the number of wave quartets (0 = choose)
 int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, const Epilogue& epi, void* accum,
-                size_t accum_bytes, int m, int n, int k, int groups, unsigned tune, hipStream_t stream) {
-    const TilePlan plan = tile_plan(m, n, k, (int)(tune & 0xffu), (int)((tune >> 8) & 0xfu), (int)((tune >> 12) & 0x3u));
-    if (plan.splits > 1 && (!accum || accum_bytes < (size_t)m * n * sizeof(unsigned long long)))
+                size_t accum_bytes, void* part, size_t part_bytes, int m, int n, int k, int groups, unsigned tune,
+                hipStream_t stream) {
+    const TilePlan plan = tile_plan_tuned(m, n, k, tune);
+    if (plan.splits > 1 && (!accum || accum_bytes < tile_accum_bytes(m, n, k, tune) || !part ||
+                            part_bytes < tile_part_bytes(m, n, k, tune)))
         return UNIQL_E_WORKSPACE;
     TileArgs a;
+    a.part = reinterpret_cast<float*>(part);
     a.B = reinterpret_cast<const u32x4*>(B);
     a.S = reinterpret_cast<const half_t*>(S);
     a.X = reinterpret_cast<const half_t*>(A);

@@ -96,6 +96,14 @@ def reset_accumulators() -> None:
     _accum_in_capture.clear()
 
 
+def _workspace(lib, m: int, n: int, k: int, k_in: int, had_block: int, flags: int):
+    """(accum bytes, temp bytes) of one layer call with these flags."""
+    acc, tmp = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    _capi.check(lib.uniql_w4a16_linear_workspace(m, n, k, k_in, had_block, flags, ctypes.byref(acc), ctypes.byref(tmp)),
+                "uniql_w4a16_linear_workspace")
+    return acc.value, tmp.value
+
+
 def _require_gpu(t: torch.Tensor, name: str) -> None:
     if not t.is_cuda:
         raise RuntimeError(f"{name} must be a GPU tensor (this package has no CPU path)")
@@ -137,12 +145,11 @@ def w4a16_gemm_ex(A: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: 
             flags |= _capi.F_TRANSPOSE_OUT
         else:
             D = torch.empty((size_m, size_n), dtype=out_dtype, device=dev)
-        need_acc = lib.uniql_w4a16_gemm_accum_bytes(size_m, size_n, size_k)
-        accum = _accumulator(dev, need_acc) if need_acc else None
-        need_tmp = lib.uniql_w4a16_gemm_temp_bytes(size_m, size_n, size_k, had_block)
-        temp = torch.empty(need_tmp, dtype=torch.uint8, device=dev) if need_tmp else None
         if out_f32:
             flags |= _capi.F_OUT_F32
+        need_acc, need_tmp = _workspace(lib, size_m, size_n, size_k, size_k, had_block, flags)
+        accum = _accumulator(dev, need_acc) if need_acc else None
+        temp = torch.empty(need_tmp, dtype=torch.uint8, device=dev) if need_tmp else None
         lda = A.stride(0) if size_m > 1 else size_k
         code = lib.uniql_w4a16_gemm(
             A.data_ptr(), lda, B.data_ptr(), s.data_ptr(), D.data_ptr(),
@@ -215,12 +222,11 @@ def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: t
             raise RuntimeError("out must be a [m, out_features] view with unit inner stride on x's device")
         if m == 0:
             return out
-        need_acc = lib.uniql_w4a16_gemm_accum_bytes(m, size_n, size_k)
-        accum = _accumulator(dev, need_acc) if need_acc else None
-        need_tmp = lib.uniql_w4a16_linear_temp_bytes(m, size_n, size_k, k_in, had_block)
-        temp = torch.empty(need_tmp, dtype=torch.uint8, device=dev) if need_tmp else None
         if out_f32:
             flags |= _capi.F_OUT_F32
+        need_acc, need_tmp = _workspace(lib, m, size_n, size_k, k_in, had_block, flags)
+        accum = _accumulator(dev, need_acc) if need_acc else None
+        temp = torch.empty(need_tmp, dtype=torch.uint8, device=dev) if need_tmp else None
         lda = x.stride(0) if m > 1 else max(k_in + (-k_in) % 8, 8)
         ldd = out.stride(0) if m > 1 else n_out
         code = lib.uniql_w4a16_linear(
