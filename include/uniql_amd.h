@@ -74,16 +74,19 @@ int uniql_stream_capture_id(void* stream, unsigned long long* id);
  *              lock array).  Only its length is checked (>= n/128, as the reference
  *              checks it); it is never read or written, so it stays zero.
  *   accum      device, uniql_w4a16_gemm_accum_bytes(m, n, k) bytes, ALL ZERO on entry
- *              and all zero again when the kernels have finished: 64-bit sum|count
- *              words through which workgroups that share an output column combine
- *              their partial sums (replaces the reference's per-call fp16 `C`
- *              buffer and its locks, marlin_gemm_kernel.cuh:515-570,1018).  A caller
- *              clears it once and reuses it for every call on the same stream; two
- *              calls that may run concurrently need separate buffers.  May be NULL
- *              when the size is 0.
+ *              and all zero again when the kernels have finished: the words through
+ *              which workgroups that share output columns combine their partial sums
+ *              (streaming kernel: a 64-bit sum|count word per output element of up to
+ *              16 rows; tiled kernel: an arrival count per output tile).  Replaces the
+ *              reference's per-call fp16 `C` buffer and its locks
+ *              (marlin_gemm_kernel.cuh:515-570,1018).  A caller clears it once and
+ *              reuses it for every call on the same stream; two calls that may run
+ *              concurrently need separate buffers.  May be NULL when the size is 0.
  *   temp       device, uniql_w4a16_gemm_temp_bytes(m, n, k, had_block) bytes, contents
- *              irrelevant (rotated activations whenever the rotation is not fused);
- *              may be NULL when that size is 0
+ *              irrelevant: rotated activations whenever the rotation is not fused, and
+ *              the fp32 partial tiles of the tiled kernel when its plan splits K over
+ *              workgroups; may be NULL when that size is 0.  Two calls that may run
+ *              concurrently need separate buffers.
  *   had_block  0: none.  Otherwise the activations are rotated first,
  *              A <- fp16(A . H_had_block * had_scale) on consecutive
  *              had_block-wide pieces of each row: 128 is fused into the
@@ -92,8 +95,10 @@ int uniql_stream_capture_id(void* stream, unsigned long long* id);
  *              kernel into `temp` first.
  *   k % 128 == 0, n % 128 == 0 (the module pads n to 256).
  *
- * Partial sums that meet in `accum` are rounded to multiples of 2^-24 and clamped to
- * +-2^22 (far beyond the fp16 range of D); NaN partials are not propagated through it.
+ * Partial sums that meet in the streaming kernel's `accum` words are rounded to multiples of
+ * 2^-24 and clamped to +-2^22 (far beyond the fp16 range of D); NaN partials are not propagated
+ * through them.  Either kernel's result is the same from run to run: integer additions in the
+ * first, partial tiles added in split order in the second.
  */
 size_t uniql_w4a16_gemm_accum_bytes(int m, int n, int k);
 size_t uniql_w4a16_gemm_temp_bytes(int m, int n, int k, int had_block);
