@@ -135,7 +135,8 @@ def test_tile_kernel_k_splits(gpu, splits):
 
 
 @pytest.mark.parametrize("m,k,n,splits,mt", [(1024, 1024, 4096, 4, 1), (1000, 1536, 2048, 3, 2), (257, 1536, 768, 3, 0),
-                                             (300, 2048, 640, 4, 4)])
+                                             (300, 2048, 640, 4, 4), (200, 640, 1280, 3, 0), (300, 896, 1280, 2, 1),
+                                             (200, 384, 1152, 3, 1)])
 def test_tile_split_exchange_is_ordered(gpu, m, k, n, splits, mt):
     """K split over workgroups of the tiled kernel: partial tiles go through scratch memory and
     the last workgroup of a tile adds them.  The result must not depend on which workgroup that
@@ -148,11 +149,15 @@ def test_tile_split_exchange_is_ordered(gpu, m, k, n, splits, mt):
     flags = F_FORCE_TILED | (splits << 8) | (mt << 16)
     first = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k, out_f32=True, flags=flags)
     assert np.abs(first.cpu().numpy() - reference_product(p, exact=True)).max() < 3e-4
+    from uniql_amd import _capi
+    _, scratch_bytes = ops._workspace(_capi.load(), m, n, k, k, 0, flags | _capi.F_OUT_F32)
+    assert scratch_bytes > 0
     same = torch.ones((), dtype=torch.bool, device=gpu)
     for rep in range(300):  # up to 4096 workgroups per call: about a million tile exchanges in all
-        if rep % 10 == 0:   # dirty what the allocator hands out next as scratch area
-            junk = torch.full((splits * m * n + 4096,), float("nan"), dtype=torch.float32, device=gpu)
-            del junk
+        # dirty the block the allocator will hand out as scratch area (same size, freed last): a
+        # slot that is read before it is written then shows as NaN
+        junk = torch.full((scratch_bytes,), 0xFF, dtype=torch.uint8, device=gpu)
+        del junk
         again = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k, out_f32=True, flags=flags)
         same &= (first == again).all()
     assert bool(same)
