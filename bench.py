@@ -176,9 +176,10 @@ def sweep(dev, gen, out_path):
     from uniql_amd import ops
     rows = []
 
-    def bench_linear(name, k, n, m, had_block=0, steps=200):
+    def bench_linear(name, k, n, m, had_block=0, steps=200, copies=None):
         per = linear_bytes(m, k, n)
-        copies = copies_for(k * n // 2) if m <= 64 else 2
+        if copies is None:
+            copies = copies_for(k * n // 2) if m <= 64 else 2
         layer = Layer(name, k, n, m, copies, dev, gen, had_block)
         sec, _ = time_graphs(lambda i: layer.run(i), copies, steps, max(20, steps // 2))
         row = dict(op=name, m=m, k=k, n=n, had_block=had_block, us=sec * 1e6, gbs=per / sec / 1e9,
@@ -194,6 +195,10 @@ def sweep(dev, gen, out_path):
     for m in (1, 2, 4, 8):
         for name, k, n in LLAMA_DECODE:
             bench_linear(name, k, n, m)
+    # the same launches over ONE copy of the weights: they stay in the 256 MB last-level cache
+    # between steps, which a model of several GB never sees; reported beside the cold numbers only
+    for name, k, n in LLAMA_DECODE:
+        bench_linear(name + "_cache_resident", k, n, 1, copies=1)
     for m in (256, 1024, 4096):
         for name, k, n in LLAMA_DECODE:
             bench_linear(name, k, n, m, steps=100)
