@@ -18,10 +18,13 @@ Pinning status (what proves each function right, besides reading):
   * group-128 quantiser (code selection) ..... golden vectors
   * dequant fp16_rn((q-8)*s) ................. closed form, exhaustive in tests
   * dequant + matmul ......................... brute-force loops on tiny shapes
-  * embedding quantise/pack/lookup ........... hand-computed tiny cases +
-    brute-force; the reference module cannot be imported without its compiled
-    extension, so `embedding_quantize`'s code selection at exact rounding ties
-    is "parity unpinned" beyond those cases
+  * embedding quantise/pack/lookup ........... hand-computed cases + brute force.  The
+    reference module cannot be imported without its compiled extension, so
+    `embedding_quantize`'s code selection is pinned by rows worked out by hand where the
+    rounding steps decide: halves (round to even), sums that only tie after the fp16
+    rounding of `w / scale + 8`, a quotient whose own fp16 rounding moves the code, the
+    same rows in float32 (different codes), the clamp, and an all-zero row
+    (tests/test_oracle_golden.py::test_embedding_quantize_rounding_ties_by_hand)
   * module forward with its fp16 roundings, SiLU-gated and squared-ReLU MLP fronts
     (linear_forward_fp16, silu_fp16, mlp_gate_up, relu2_fp16) ... torch's own fp16 CPU
     operators over all finite fp16 inputs / random tensors (the reference calls exactly

@@ -95,6 +95,12 @@ def test_argument_checks_need_no_gpu(lib):
     assert call(ldd=4095) == -2
     assert call(flags=8, ldd=0) == -2                    # transposed: ldd counts rows
     assert call(m=0) == 0
+    # the tiled kernel addresses a tile's X rows with 32-bit byte offsets from the tile's first
+    # row: a row stride of 2^24 elements or more is refused before anything is enqueued (the
+    # pointers are never dereferenced: the shape check comes first)
+    fake = ctypes.c_void_p(0x10000)
+    assert call(A=fake, B=fake, S=fake, D=fake, m=17, n=128, k=128, k_in=128, groups=1, ldd=128, n_out=128,
+                lda=1 << 24) == -2
     assert lib.uniql_w4a16_linear_temp_bytes(3, 4096, 4096, 4000, 0) == 3 * 4096 * 2
     assert lib.uniql_w4a16_linear_temp_bytes(3, 4096, 4096, 4096, 0) == 0
     r = lib.uniql_rope_indices

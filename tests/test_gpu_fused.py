@@ -58,10 +58,8 @@ def test_cut_and_bias_equal_the_unfused_sequence(gpu, m, k, n, n_out):
     # products sit on either side of a power of two) survives the bias add, whose own rounding
     # can add a step at the sum's magnitude
     step = 8 * fp16_half_ulp(np.maximum(np.abs(prod.astype(np.float64)), np.abs(want.astype(np.float64))))
-    if m > 16:   # the tiled kernel multiplies the reference's fp16-rounded weights: same roundings throughout
-        assert (diff <= step).all() and (diff > 0).mean() < 5e-3
-    else:        # the streaming kernel's unrounded weights move the product by up to 1e-4 sqrt(k)
-        assert (diff <= 1e-4 * np.sqrt(k) + step).all()
+    # both kernels multiply the reference's fp16-rounded weights: same roundings throughout
+    assert (diff <= step).all() and (diff > 0).mean() < 5e-3
 
 
 @pytest.mark.parametrize("m", [1, 3, 16, 17, 100, 256])

@@ -217,6 +217,23 @@ def test_deterministic_and_repeatable(gpu):
     assert np.array_equal(a.view(np.uint16), b.view(np.uint16))
 
 
+@pytest.mark.parametrize("m", [1, 3])
+def test_nan_propagates_with_and_without_k_split(gpu, m):
+    """A NaN activation makes its row NaN whether or not the launch splits K over workgroups
+    (the partial sums then meet in the fixed-point accumulator words, which carry a NaN
+    count); other rows are untouched, and the accumulator words are zero again afterwards."""
+    p = make_linear_problem(m, 4096, 512, seed=90 + m)
+    p["x"][m - 1, 1000] = np.nan
+    split = run_gemm(p, gpu, out_f32=True)                        # 32 groups over several workgroups
+    whole = run_gemm(p, gpu, out_f32=True, flags=(8 << 8) | (4 << 16))   # 4 waves x 8 groups: one workgroup per strip
+    for y in (split, whole):
+        assert np.isnan(y[m - 1]).all()
+        assert np.isfinite(y[:m - 1]).all()
+    assert np.array_equal(split[:m - 1], whole[:m - 1]) or np.abs(split[:m - 1] - whole[:m - 1]).max() < 1e-5
+    y16 = run_gemm(p, gpu)
+    assert np.isnan(y16[m - 1]).all()
+
+
 def test_row_stride(gpu):
     """A may be a row-strided view (lda > k)."""
     from uniql_amd import ops
@@ -457,7 +474,7 @@ def test_lm_head_shape(gpu, m):
     ref = (x.float() @ w.float()).cpu().numpy()
     del w
     y32 = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k, out_f32=True).cpu().numpy()
-    assert np.abs(y32 - ref).max() < (1e-4 * np.sqrt(k) + 2e-4 if m <= 16 else 5e-4)
+    assert np.abs(y32 - ref).max() < 5e-4
     y = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k)
     assert np.array_equal(y.cpu().numpy(), y32.astype(np.float16))
     check_layer_output(y.cpu().numpy(), ref)

@@ -106,6 +106,25 @@ def test_embedding_quantize_bit_exact(gpu, v, d):
     assert np.array_equal(packed.cpu().numpy(), np.asarray(o_packed))
 
 
+def test_embedding_quantize_hand_computed_ties(gpu):
+    """The device quantiser on the rows whose codes are worked out by hand in
+    tests/test_oracle_golden.py::test_embedding_quantize_rounding_ties_by_hand (fp16 rounding of
+    every step, halves to even, clamp, all-zero row): literal expectations, no oracle call."""
+    from uniql_amd import ops
+    rows = torch.tensor([[8.0, 0.5, 1.5, -0.5, -1.5, 2.5, 257 / 512, -257 / 512],
+                         [7.0, 1341 / 1024, 1340 / 1024, 0.4375, -7.0, 0.0, 0.0, 0.0],
+                         [0.0] * 8], dtype=torch.float16)
+    packed, scales = ops.w4_embedding_quantize(rows.to(gpu))
+    assert scales.cpu().tolist() == [1.0, 0.875, 0.0]
+    want = [[15, 8, 10, 8, 6, 10, 8, 8], [15, 10, 9, 8, 0, 8, 8, 8], [0] * 8]
+    words = packed.cpu().numpy().view(np.uint32)[:, 0]
+    for r in range(3):
+        got = [0] * 8
+        for i, e in enumerate([0, 2, 4, 6, 1, 3, 5, 7]):      # nibble i holds element e
+            got[e] = int(words[r] >> np.uint32(4 * i)) & 15
+        assert got == want[r], (r, got)
+
+
 def test_embedding_module_from_fp16_on_the_device(gpu):
     from uniql_amd.quantize.quant_embedding_layers import W4O16Embedding
     emb = torch.nn.Embedding(500, 512).half()

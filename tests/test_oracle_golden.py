@@ -194,6 +194,46 @@ def test_embedding_hand_case():
     assert out[0].tolist() == [-8.0, -3.0, 0.0, 7.0, 1.0, 2.0, -1.0, 7.0]
 
 
+def _emb_codes(row, dtype):
+    packed, scales = O.embedding_quantize(torch.tensor([row], dtype=dtype))
+    return O.embedding_unpack(packed)[0].tolist(), scales.tolist()
+
+
+def test_embedding_quantize_rounding_ties_by_hand():
+    """Code selection of W4O16Embedding.from_fp16 (quant_embedding_layers.py:35-37) where the
+    rounding steps decide, worked out by hand (not by running the oracle's formula again):
+    every operation rounds in the WEIGHT's dtype, and torch.round rounds halves to even.
+
+    Row A, max |w| = 8 -> scale 1 (division exact), fp16:
+      0.5 -> 8.5 -> 8;  1.5 -> 9.5 -> 10;  -0.5 -> 7.5 -> 8;  -1.5 -> 6.5 -> 6;  2.5 -> 10.5 -> 10
+      257/512 = 0.501953125: the sum 8.501953125 lies between the fp16 neighbours 8.5 and 8.5078125
+      (spacing 2^-7 in [8, 16)) and rounds to 8.5, a tie that appears only in fp16 -> 8; in
+      float32 the sum is exact and rounds to 9.  -257/512: 7.498046875 -> fp16 7.5 -> 8; float32 -> 7.
+      8.0 -> 16 -> clamped to 15.
+    Row B, max |w| = 7 -> scale 0.875, fp16: 1341/1024 / 0.875 = 1.496652 rounds to the fp16
+      quotient 1533/1024 = 1.4970703 (neighbour 1532/1024 is farther: 0.000558 against 0.000418);
+      + 8 = 9.4970703 lies between 9.4921875 and 9.5 and rounds to 9.5 (0.0029 against 0.0049)
+      -> 10, while exact arithmetic gives round(9.496652) = 9 (float32 does).
+      1340/1024: quotient 1.4955357 -> 1531/1024 = 1.4951172; + 8 -> 9.4921875 -> 9 in both.
+      0.4375 / 0.875 = 0.5 exactly -> 8.5 -> 8;  -7 -> -8 + 8 = 0.
+    Row C, all zero: scale 0, 0/0 = NaN, NaN survives round and clamp, the int32 conversion
+      gives 0x80000000 whose low nibble is 0 -> code 0 (and the lookup returns -0.0 = -8 * 0)."""
+    row_a = [8.0, 0.5, 1.5, -0.5, -1.5, 2.5, 257 / 512, -257 / 512]
+    codes, scales = _emb_codes(row_a, torch.float16)
+    assert scales == [1.0] and codes == [15, 8, 10, 8, 6, 10, 8, 8]
+    codes, _ = _emb_codes(row_a, torch.float32)
+    assert codes == [15, 8, 10, 8, 6, 10, 9, 7]
+    row_b = [7.0, 1341 / 1024, 1340 / 1024, 0.4375, -7.0, 0.0, 0.0, 0.0]
+    codes, scales = _emb_codes(row_b, torch.float16)
+    assert scales == [0.875] and codes == [15, 10, 9, 8, 0, 8, 8, 8]
+    codes, _ = _emb_codes(row_b, torch.float32)
+    assert codes == [15, 9, 9, 8, 0, 8, 8, 8]
+    packed, scales = O.embedding_quantize(torch.zeros(1, 16, dtype=torch.float16))
+    assert scales.tolist() == [0.0] and O.embedding_unpack(packed)[0].tolist() == [0] * 16
+    out = O.embedding_lookup(np.array([0]), packed, scales)
+    assert np.array_equal(out.view(np.uint16), np.full((1, 16), 0x8000, dtype=np.uint16))
+
+
 def test_embedding_roundtrip_and_gather():
     g = torch.Generator().manual_seed(2)
     w = torch.randn(50, 64, generator=g).to(torch.float16)

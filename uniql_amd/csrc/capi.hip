@@ -11,6 +11,7 @@ int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* 
                 size_t accum_bytes, void* part, size_t part_bytes, int m, int n, int k, int groups, unsigned tune,
                 hipStream_t stream);
 size_t tile_part_bytes(int m, int n, int k, unsigned tune);
+bool tile_shape_ok(int m, int n, int k, int64_t ldx, unsigned tune);
 int pad_rows_launch(const void* A, int64_t lda, int k_in, void* dst, int k, int m, hipStream_t stream);
 size_t tile_accum_bytes(int m, int n, int k, unsigned tune = 0);
 int dequant_launch(const void* B, const void* S, void* W, uint8_t* codes, int n, int k, int groups,
@@ -174,6 +175,8 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
     const size_t part_bytes = use_stream ? 0 : tile_part_bytes(m, n, k, tune);
     if (act_bytes + part_bytes > 0 && (!temp || temp_bytes < act_bytes + part_bytes)) return UNIQL_E_WORKSPACE;
     void* part = part_bytes ? reinterpret_cast<char*>(temp) + act_bytes : nullptr;
+    // last check before the first kernel is enqueued: whether the tiled kernel can take the shape
+    if (!use_stream && !tile_shape_ok(m, n, k, (rotate_first || pad_first) ? (int64_t)k : lda, tune)) return UNIQL_E_SHAPE;
     if (pad_first) {
         const int e = pad_rows_launch(A, lda, k_in, temp, k, m, st);
         if (e != UNIQL_OK) return e;

@@ -154,25 +154,35 @@ __device__ __forceinline__ void finish_store_gated(const Epilogue& e, void* D, i
 }
 
 // ---- exchange of partial sums between workgroups that split K ------------------------
-// One 64-bit word per output element in a zero-initialised buffer: bits 8..63 the running sum
-// in units of 2^-24, bits 0..7 the number of contributions.  Integer adds commute, so the total
-// does not depend on arrival order.
+// One 64-bit word per output element in a zero-initialised buffer:
+//   bits 14..63  the running sum in units of 2^-24 (two's complement, 50 bits),
+//   bits  7..13  the number of contributions that were NaN,
+//   bits  0..6   the number of contributions.
+// Integer adds commute, so the total does not depend on arrival order.  A contribution is
+// clamped to +-2^18 (beyond the fp16 range of the output, so an infinite partial sum still
+// gives an infinite fp16 result) and at most 127 contributions meet in a word: the sum
+// field cannot overflow into nothing, the counts cannot carry into the sum.  A NaN partial
+// sum adds nothing to the sum and one to the NaN count; the total then reads as NaN, as it
+// would without a K split.
 constexpr float kAccumScale = 16777216.0f;  // 2^24 fixed-point units per 1.0
-constexpr float kAccumClamp = 4194304.0f;   // 2^22: far beyond the fp16 range of the outputs
+constexpr float kAccumClamp = 262144.0f;    // 2^18
+constexpr int kAccumMaxSplits = 127;
 
 __device__ __forceinline__ unsigned long long accum_word(float v, unsigned count) {
-    const float c = fminf(fmaxf(v, -kAccumClamp), kAccumClamp);
-    return ((unsigned long long)__float2ll_rn(c * kAccumScale) << 8) + count;
+    const bool is_nan = v != v;
+    const float c = is_nan ? 0.f : fminf(fmaxf(v, -kAccumClamp), kAccumClamp);
+    return ((unsigned long long)__float2ll_rn(c * kAccumScale) << 14) + (is_nan ? 128u : 0u) + count;
 }
 __device__ __forceinline__ float accum_value(unsigned long long word) {
-    return (float)((long long)word >> 8) * (1.0f / kAccumScale);
+    const float v = (float)((long long)word >> 14) * (1.0f / kAccumScale);
+    return (word & 0x3f80ull) ? __builtin_nanf("") : v;
 }
 // Adds one contribution.  True for the last of `splits` arrivals, which gets the total and
 // must put the word back to zero (accum_reset) after using it.
 __device__ __forceinline__ bool accum_add(unsigned long long* p, float v, int splits, float& total) {
     const unsigned long long word = accum_word(v, 1u);
     const unsigned long long old = __hip_atomic_fetch_add(p, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if ((int)(old & 0xffull) != splits - 1) return false;
+    if ((int)(old & 0x7full) != splits - 1) return false;
     total = accum_value(old + word);
     return true;
 }
@@ -193,7 +203,7 @@ __device__ __forceinline__ bool accum_add_pair(unsigned long long* pg, unsigned 
     asm volatile("" : "+v"(lo) : "v"(returned));  // the gate word now depends on the up add's return value
     word = (word & 0xffffffff00000000ull) | lo;
     const unsigned long long old = __hip_atomic_fetch_add(pg, word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if ((int)(old & 0xffull) != splits - 1) return false;
+    if ((int)(old & 0x7full) != splits - 1) return false;
     total_g = accum_value(old + word);
     total_u = accum_value(__hip_atomic_exchange(pu, 0ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
     return true;

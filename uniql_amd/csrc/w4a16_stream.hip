@@ -15,27 +15,23 @@
 // used purely as a wide dot-product unit: its cost does not depend on M, so
 // M = 1..16 all run at the weight-streaming rate.
 //
-// Expanding codes to scaled fp16 weights costs 13 vector instructions per packed
-// word, which at M <= 16 is more vector work than the memory system leaves time for.
-// This kernel feeds the RAW codes to the matrix unit instead:
-//   * `word & 0x000f000f` read as two fp16 values is (code * 2^-24) twice: a
-//     subnormal, which the MFMA unit multiplies exactly.  `word & 0x00f000f0` is
-//     (16 code * 2^-24); the matching activations are staged pre-divided by 16.
-//     Five instructions per packed word (one shift, four ANDs).
-//   * the zero point: sum_k x_k (code_k - 8) = sum_k x_k code_k - 8 sum_k x_k.  The
-//     second term only depends on the activation row and the group; it is computed
-//     once while staging and enters the group's first MFMA as its C operand.
-//   * the scale multiplies the group's fp32 dot product (one FMA per output and
-//     group) instead of every weight.
-// The result is sum_g s_g . sum_k x_k (code_k - 8) with fp32 arithmetic throughout:
-// the same value as the reference's up to its fp16 rounding of every scaled weight.
+// Every weight is expanded to the reference's fp16 value fp16_rn((code - 8) * scale)
+// (csrc/linear/marlin_gemm_kernel.cuh:118-146) before it enters the matrix unit: 13 vector
+// instructions per packed word (one shift, four mask-and-or, two fp16 subtractions, two fp16
+// fused multiply-adds, four fp16 multiplications by the scale), all exact except the final
+// multiplication, which rounds once as the reference's does.  The products are exact in the
+// MFMA and accumulate in fp32, so the result equals the reference's value up to the order of
+// the fp32 additions, for every M.  (Feeding the raw codes as fp16 subnormals and scaling each
+// group's fp32 dot product instead saves 8 of the 13 instructions, but leaves out the fp16
+// rounding of the scaled weights: up to 5e-3 away from the reference's value at K = 14336,
+// which an fp16 output between 16 and 32 cannot absorb inside a max-abs tolerance of 1e-2.)
 //
 // Work split: unit = (strip of 128 columns) x (group of 128 K).  A wave owns `upw`
 // consecutive groups of a strip, the four or eight waves of a workgroup own consecutive
 // group ranges, partial sums meet in LDS.  When K is split over several workgroups,
-// each output element has a 64-bit word in a zero-initialised accumulator: bits 8..63
-// hold the running sum as a fixed-point integer (2^-24 units), bits 0..7 the number of
-// contributions.  A workgroup adds (value << 8) + 1 with ONE device-scope atomic and
+// each output element has a 64-bit word in a zero-initialised accumulator: bits 14..63
+// hold the running sum as a fixed-point integer (2^-24 units), bits 7..13 the number of NaN
+// contributions, bits 0..6 the number of contributions.  A workgroup adds (value << 14) + 1 with ONE device-scope atomic and
 // looks at the returned old word: whoever sees count == splits - 1 was last, owns the
 // total (old + own), stores the output and writes the word back to zero.  Integer adds
 // commute, so the result does not depend on arrival order, and nobody waits for anyone.
@@ -104,26 +100,21 @@ void w4a16_stream_kernel(const StreamArgs a) {
     const u32x4* strip_w = a.B + (size_t)strip * 64;
     const half_t* strip_s = a.S + (size_t)strip * 128;
 
-    float acc[8][NV];
+    f4 acc[8];  // acc[jb][v]: output row 4 kq + v, column slot jb of this lane
 #pragma unroll
-    for (int jb = 0; jb < 8; ++jb)
-#pragma unroll
-        for (int v = 0; v < NV; ++v) acc[jb][v] = 0.f;
+    for (int jb = 0; jb < 8; ++jb) acc[jb] = f4{0.f, 0.f, 0.f, 0.f};
 
     uint32_t* xs = lds + (size_t)w * a.xrows * kXsStride;  // this wave's staging rows
     // Staged row layout (dwords): the pair of K values 2d, 2d+1 of the group, d = 16 rp + kq' + 4 t,
     // sits at dword 16 rp + 4 kq' + t, so that the A operand of lane (row, kq') for row pair rp
-    // is one 16-byte read; pairs with odd t (K rows 8..15 of a packed row) are stored divided
-    // by 16.  Dword 64 of the row holds 8 * 2^-24 * (sum of the row's values) as fp32.
+    // is one 16-byte read.
     // MFMA row `slot` reads staged row min(slot, xrows - 1): rows past M only feed output rows
     // that are never stored.
     const int xrow_of = (slot < a.xrows ? slot : a.xrows - 1) * kXsStride + 4 * kq;
     // where this lane's staged quad goes: lane `slot` holds pairs d = 4 slot + i
     const int stage_off = 16 * (slot >> 2) + (slot & 3);
-    const half_t stage_mul = (slot & 1) ? (half_t)0.0625f : (half_t)1.0f;
-    const h2 stage_mul2 = h2{stage_mul, stage_mul};
-    uint32_t mask_low = 0x000f000fu, mask_high = 0x00f000f0u;
-    asm volatile("" : "+s"(mask_low), "+s"(mask_high));  // keep both masks in scalar registers
+    NibbleMagic magic;
+    magic.init();
 
     u32x4 wq[2 * RPW];
     u32x4 sc;
@@ -181,19 +172,9 @@ void w4a16_stream_kernel(const StreamArgs a) {
                         v[p] = h2_to_bits(hv);
                     }
                 }
-                // 8 * 2^-24 * (sum of the row), from the values the MFMA will see
-                float sum = 0.f;
-#pragma unroll
-                for (int p = 0; p < 4; ++p) {
-                    const h2 hv = bits_to_h2(v[p]);
-                    sum += (float)hv.x + (float)hv.y;
-                }
-#pragma unroll
-                for (int d = 1; d < 16; d <<= 1) sum += __shfl_xor(sum, d, kWave);
                 uint32_t* row = xs + (size_t)(mrow + kq) * kXsStride;
 #pragma unroll
-                for (int p = 0; p < 4; ++p) row[stage_off + 4 * p] = h2_to_bits(bits_to_h2(v[p]) * stage_mul2);
-                if (slot == 0) reinterpret_cast<float*>(row)[64] = sum * (8.0f / kAccumScale);
+                for (int p = 0; p < 4; ++p) row[stage_off + 4 * p] = v[p];
             }
         }
         // LDS operations of one wave complete in issue order: the reads below see
@@ -204,47 +185,28 @@ void w4a16_stream_kernel(const StreamArgs a) {
 
         const u32x4 (&cur)[2 * RPW] = wq;
         const u32x4 sc_cur = sc;
-        h8 xa[RPW];
-        f4 zp;  // minus 8 * row sums for this lane's four output rows: the first MFMA's C operand
+        // Row pair rp (packed rows 2rp, 2rp+1 = 32 K values) against the eight column slots
+        // jb = 2j + blk of this lane: the B operand is the four code pairs of words j of both
+        // packed rows (low byte pair for blk 0, after >> 8 for blk 1), expanded and scaled; the
+        // scale of column slot jb is half jb of the 16-byte scale load.  Consecutive MFMAs go to
+        // different accumulators.
 #pragma unroll
-        for (int rp = 0; rp < RPW; ++rp)
-            xa[rp] = __builtin_bit_cast(h8, *reinterpret_cast<const u32x4*>(xs + xrow_of + 16 * rp));
+        for (int rp = 0; rp < RPW; ++rp) {
+            const h8 xa = __builtin_bit_cast(h8, *reinterpret_cast<const u32x4*>(xs + xrow_of + 16 * rp));
 #pragma unroll
-        for (int v = 0; v < 4; ++v) {
-            const int r = 4 * kq + v;
-            const float* sums = reinterpret_cast<const float*>(xs) + (r < a.xrows ? r : a.xrows - 1) * kXsStride + 64;
-            zp[v] = (v >= NV) ? 0.f : -sums[0];
-        }
-        // two passes over the columns (word pairs j) keep the group's raw dot products in
-        // sixteen registers; the scale of output column jb of this lane is half jb of the
-        // 16-byte scale load
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t q0 = cur[2 * rp][j], q1 = cur[2 * rp + 1][j];
+                const h2 pr = bits_to_h2(sc_cur[j]);
 #pragma unroll
-        for (int jh = 0; jh < 2; ++jh) {
-            f4 dot[4];
-#pragma unroll
-            for (int rp = 0; rp < RPW; ++rp) {
-#pragma unroll
-                for (int jl = 0; jl < 2; ++jl) {
-                    const int j = 2 * jh + jl;
-                    const uint32_t q0 = cur[2 * rp][j], q1 = cur[2 * rp + 1][j];
-#pragma unroll
-                    for (int blk = 0; blk < 2; ++blk) {
-                        const uint32_t p0 = blk ? (q0 >> 8) : q0;
-                        const uint32_t p1 = blk ? (q1 >> 8) : q1;
-                        const u32x4 raw = u32x4{p0 & mask_low, p0 & mask_high, p1 & mask_low, p1 & mask_high};
-                        const h8 bw = __builtin_bit_cast(h8, raw);
-                        dot[2 * jl + blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(
-                            xa[rp], bw, rp == 0 ? zp : dot[2 * jl + blk], 0, 0, 0);
-                    }
+                for (int blk = 0; blk < 2; ++blk) {
+                    const uint32_t p0 = blk ? (q0 >> 8) : q0;
+                    const uint32_t p1 = blk ? (q1 >> 8) : q1;
+                    const h2 sv = blk ? h2{pr.y, pr.y} : h2{pr.x, pr.x};
+                    const h2 e0 = magic.pair_low(p0) * sv, e1 = magic.pair_high(p0) * sv;
+                    const h2 e2 = magic.pair_low(p1) * sv, e3 = magic.pair_high(p1) * sv;
+                    const h8 bw = h8{e0.x, e0.y, e1.x, e1.y, e2.x, e2.y, e3.x, e3.y};
+                    acc[2 * j + blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, bw, acc[2 * j + blk], 0, 0, 0);
                 }
-            }
-#pragma unroll
-            for (int jq = 0; jq < 4; ++jq) {
-                const int jb = 4 * jh + jq;
-                const h2 pr = bits_to_h2(sc_cur[jb >> 1]);
-                const float sf = (float)((jb & 1) ? pr.y : pr.x);
-#pragma unroll
-                for (int v = 0; v < NV; ++v) acc[jb][v] += dot[jq][v] * sf;
             }
         }
     }
@@ -280,7 +242,7 @@ void w4a16_stream_kernel(const StreamArgs a) {
                     const int ml = 4 * kq + v;
                     if (ml < a.M)
                         red[((w % wpr) * rr_rows + ml) * 128 + ncol_lane + 16 * (jb >> 1) + 8 * (jb & 1)] =
-                            acc[jb][v] * kAccumScale;
+                            acc[jb][v];
                 }
             }
         }
@@ -371,7 +333,7 @@ static StreamPlan stream_plan(int m, int n, int k, int upw_override, int waves_o
         while (p.upw < 8 && (int64_t)nstrips * ceil_div(G, p.waves * p.upw) > max_wgs) p.upw *= 2;
     }
     p.splits = ceil_div(G, p.waves * p.upw);
-    while (p.splits > 255) {  // the contribution count has 8 bits
+    while (p.splits > kAccumMaxSplits) {  // the contribution count has 7 bits
         p.upw *= 2;
         p.splits = ceil_div(G, p.waves * p.upw);
     }

@@ -31,8 +31,10 @@
 // vmcnt is counted by hand: every stage issues exactly kStageOps LDS-DMA operations per
 // wave and nothing else uses the counter inside the loop.
 //
-// When K is also split over workgroups the tile goes through the same 64-bit fixed-point
-// sum|count words as the streaming kernel.
+// When K is also split over workgroups every workgroup writes its fp32 partial tile to a scratch
+// area and the last one to arrive (one arrival count per tile) adds them in split order.
+#include <atomic>
+
 #include "common.hpp"
 
 namespace uniql {
@@ -214,14 +216,16 @@ __global__ __launch_bounds__(256 * KW, 1) void w4a16_tile_kernel(const TileArgs 
     // X tile: wave w brings rows [kXOps 4 w, kXOps 4 (w+1)); one DMA instruction covers 4 rows
     // (64 lanes x 16 bytes, contiguous in LDS).  Lane l lands at row l/16, position l%16, so
     // it must fetch segment (l % 16) ^ (row % 16) of its row.
-    uint32_t xsrc[kXOps];  // byte offsets from X + 128 g (uniform): scalar base + 32-bit lane offset addressing
+    // byte offsets from the tile's first row, X + m0 ldx + 128 g (uniform, 64-bit): scalar base +
+    // 32-bit lane offset addressing; the host keeps 128 ldx below 2^31 elements
+    uint32_t xsrc[kXOps];
+    const half_t* x_tile = a.X + (size_t)m0 * a.ldx;
 #pragma unroll
     for (int i = 0; i < kXOps; ++i) {
         const int row = kXOps * 4 * w + 4 * i + dkq;
         const int seg = dslot ^ (row & 15);
-        const int m = m0 + row;
-        const int mc = m < a.M ? m : a.M - 1;  // rows past M re-read the last row: never stored
-        xsrc[i] = (uint32_t)(((size_t)mc * a.ldx + 8 * seg) * sizeof(half_t));
+        const int rc = m0 + row < a.M ? row : a.M - 1 - m0;  // rows past M re-read the last row: never stored
+        xsrc[i] = (uint32_t)(((size_t)rc * a.ldx + 8 * seg) * sizeof(half_t));
     }
 
     NibbleMagic magic;
@@ -259,7 +263,7 @@ __global__ __launch_bounds__(256 * KW, 1) void w4a16_tile_kernel(const TileArgs 
         uint32_t* stage = lds + ring * L::kStageDwords;
         if (idx < kXOps) {
             uint32_t* xbuf = stage + (kXOps * 4 * w) * 64;  // this wave's X rows
-            const char* xg = reinterpret_cast<const char*>(a.X + 128 * g);  // uniform
+            const char* xg = reinterpret_cast<const char*>(x_tile + 128 * g);  // uniform
             __builtin_amdgcn_global_load_lds((gptr_t)(xg + xsrc[idx]), (lptr_t)(xbuf + idx * 256), 16, 0, 0);
         } else if (idx < kXOps + 2) {
             uint32_t* bbuf = stage + L::kXDwords + w * 512 + (idx - kXOps) * 256;
@@ -658,14 +662,30 @@ static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_overr
     return p;
 }
 
+// Whether tile_launch can take the call: grid size, and the 32-bit in-tile offsets of the X loads
+// (128 rows of ldx elements, 2 bytes each, must stay below 2^32).  Checked by the entry point
+// before anything is enqueued.
+bool tile_shape_ok(int m, int n, int k, int64_t ldx, unsigned tune) {
+    const TilePlan plan = tile_plan_tuned(m, n, k, tune);
+    const int64_t grid = (int64_t)(n / 128) * ceil_div_i(m, 32 * plan.mtiles) * plan.splits;
+    return grid <= 0x7fffffffLL && ldx < (1LL << 24);
+}
+
 template <int MT, bool EXT, int KW>
 static hipError_t tile_launch_one(const TileArgs& a, int grid, hipStream_t stream) {
     const size_t shmem = TileLds<MT, KW>::kBytes;
     auto kern = &w4a16_tile_kernel<MT, EXT, KW>;
     if (shmem > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-        if (e != hipSuccess) return e;
+        // the attribute is a property of (instantiation, device): set it on the first launch there
+        static std::atomic<unsigned long long> done{0};
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess) return hipErrorInvalidDevice;
+        if (dev < 0 || dev >= 64 || !((done.load(std::memory_order_relaxed) >> dev) & 1ull)) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
+            if (e != hipSuccess) return e;
+            if (dev >= 0 && dev < 64) done.fetch_or(1ull << dev, std::memory_order_relaxed);
+        }
     }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256 * KW), shmem, stream, a);
     return hipGetLastError();
