@@ -173,6 +173,21 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
                        unsigned flags, void* stream);
 
 /*
+ * Measurement aid, no counterpart in the reference: launches a kernel that only READS what the
+ * streaming kernel (m <= 16) of uniql_w4a16_gemm reads for this shape - every packed weight and
+ * scale once, with the same grid, waves per workgroup, walk over the K groups and 16-byte loads -
+ * and computes nothing.  Its duration is the floor the memory system and the launch set for that
+ * plan; bench.py reports it beside the product kernel's.
+ *   sink    device, uniql_w4a16_read_floor_sink_bytes(m, n, k, flags) bytes: practically never written
+ *   flags   the streaming kernel's tuning fields (bits 8..15, 16..20) choose the same plan;
+ *           bits 21..23: units a wave requests before it consumes the first (0 or 1: one, as the
+ *           product kernel does per register set; 2 or 4: deeper)
+ */
+size_t uniql_w4a16_read_floor_sink_bytes(int m, int n, int k, unsigned flags);
+int uniql_w4a16_read_floor(const void* B, const void* S, void* sink, size_t sink_bytes, int m, int n, int k,
+                           unsigned flags, void* stream);
+
+/*
  * W[k, n] fp16 = fp16_rn((code - 8) * scale), natural (un-permuted) order.
  * The value csrc/linear/marlin_gemm_kernel.cuh:118-146 builds in registers and
  * quantize/quantize_helpers.py:118 calls w_ref.  Also writes the raw codes

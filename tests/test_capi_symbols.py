@@ -64,6 +64,11 @@ def test_host_only_entry_points(lib):
     assert ws(1, 4096 + 64, 4096, 4096, 0, 0, ctypes.byref(acc), ctypes.byref(tmp)) == -2
     assert ws(1, 4096, 4096, 4096, 0, 0, None, ctypes.byref(tmp)) == -1
     assert lib.uniql_stream_capture_id(None, None) == -1    # the result pointer is checked before any HIP call
+    # the read-floor aid: one dword per wave of the streaming plan (o_proj at one row: 256 workgroups of 4 waves)
+    assert lib.uniql_w4a16_read_floor_sink_bytes(1, 4096, 4096, 0) == 256 * 4 * 4
+    assert lib.uniql_w4a16_read_floor_sink_bytes(1, 4096 + 64, 4096, 0) == 0
+    assert lib.uniql_w4a16_read_floor(None, None, None, 0, 1, 4096, 4096 + 16, 0, None) == -2
+    assert lib.uniql_w4a16_read_floor(None, None, None, 0, 1, 4096, 4096, 0, None) == -1
 
 
 def test_argument_checks_need_no_gpu(lib):

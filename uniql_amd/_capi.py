@@ -36,6 +36,8 @@ SIGNATURES = {
                                    c_void_p, c_int64, c_void_p, c_int64, c_int, c_int,
                                    c_void_p, c_int64, c_void_p, c_size_t, c_void_p, c_size_t,
                                    c_int, c_int, c_int, c_int, c_int, c_float, c_uint, c_void_p]),
+    "uniql_w4a16_read_floor_sink_bytes": (c_size_t, [c_int, c_int, c_int, c_uint]),
+    "uniql_w4a16_read_floor": (c_int, [c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int, c_int, c_uint, c_void_p]),
     "uniql_w4a16_dequant": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_void_p]),
     "uniql_w4a16_quantize": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
                                      c_int, c_int, c_int, c_int, c_void_p]),

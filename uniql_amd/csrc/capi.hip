@@ -7,6 +7,8 @@ int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const 
                   const Epilogue& epi, void* accum, int m, int n, int k, int groups, bool had128, float had_scale,
                   unsigned tune, hipStream_t stream);
 size_t stream_accum_bytes(int m, int n, int k);
+int read_floor_launch(const void* B, const void* S, void* sink, int m, int n, int k, unsigned tune, hipStream_t stream);
+size_t read_floor_sink_bytes(int m, int n, int k, unsigned tune);
 int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, const Epilogue& epi, void* accum,
                 size_t accum_bytes, void* part, size_t part_bytes, int m, int n, int k, int groups, unsigned tune,
                 hipStream_t stream);
@@ -215,6 +217,22 @@ int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, v
     const int64_t ldd = (flags & UNIQL_F_TRANSPOSE_OUT) ? (int64_t)((m + 7) / 8) * 8 : n;
     return uniql_w4a16_linear(A, lda, k, B, S, nullptr, nullptr, 0, D, ldd, n, UNIQL_EPI_NONE, workspace, workspace_len, accum,
                               accum_bytes, temp, temp_bytes, m, n, k, groups, had_block, had_scale, flags, stream);
+}
+
+int uniql_w4a16_read_floor(const void* B, const void* S, void* sink, size_t sink_bytes, int m, int n, int k,
+                           unsigned flags, void* stream) {
+    const int rc = check_linear_shape(m, n, k, k / 128);
+    if (rc != UNIQL_OK) return rc;
+    if (m <= 0) return UNIQL_E_SHAPE;
+    if (!B || !S || !sink) return UNIQL_E_NULL;
+    if (!aligned16(B) || !aligned16(S)) return UNIQL_E_ALIGN;
+    if (sink_bytes < read_floor_sink_bytes(m, n, k, flags >> 8)) return UNIQL_E_WORKSPACE;
+    return read_floor_launch(B, S, sink, m, n, k, flags >> 8, reinterpret_cast<hipStream_t>(stream));
+}
+
+size_t uniql_w4a16_read_floor_sink_bytes(int m, int n, int k, unsigned flags) {
+    if (m <= 0 || n <= 0 || k <= 0 || n % 128 != 0 || k % 128 != 0) return 0;
+    return read_floor_sink_bytes(m, n, k, flags >> 8);
 }
 
 int uniql_w4a16_dequant(const void* B, const void* S, void* W, uint8_t* codes, int n, int k, int groups,

@@ -65,14 +65,12 @@ struct StreamArgs {
 // (1, 2, 4, 8, 16): it fixes NV, how many of the four output rows of a lane's accumulator
 // quad are real, and XQ, how many quads of activation rows are loaded and staged.  WAVES:
 // wavefronts per workgroup (4 or 8); with 8 a workgroup can cover all of K for shapes with
-// many strips, which removes the exchange of partial sums between workgroups.  A wave keeps one
-// group's weights in registers at a time: a second register set for the next group costs more
-// in occupancy than it hides in latency, the other waves of the SIMD do that.  EXT: the call
+// many strips, which removes the exchange of partial sums between workgroups.  EXT: the call
 // uses something beyond the plain product (input shorter than K, output cut or strided, bias,
 // gated pairs); the plain instantiation leaves all of that code out, which at a few
 // microseconds per launch is measurable (instruction fetch).
 template <int RC, bool HAD, int WAVES, bool EXT>
-__global__ __launch_bounds__(64 * WAVES, 3)
+__global__ __launch_bounds__(64 * WAVES, RC == 16 ? 2 : 3)
 void w4a16_stream_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     constexpr int NV = RC < 4 ? RC : 4;
@@ -116,21 +114,26 @@ void w4a16_stream_kernel(const StreamArgs a) {
     NibbleMagic magic;
     magic.init();
 
-    u32x4 wq[2 * RPW];
-    u32x4 sc;
-    u32x4 xv[XQ];
-    // everything group g needs from memory: activations first (small, they gate the LDS
-    // staging), then scales, then the eight packed rows
-    auto issue_loads = [&](int g) {
+    // Everything a group needs from memory, held in registers: two sets, so that the loads of the
+    // wave's next group are in flight while the current one is expanded and multiplied (the
+    // expansion is about as long as the memory latency it would otherwise leave uncovered).
+    struct GroupRegs {
+        u32x4 wq[2 * RPW];
+        u32x4 sc;
+        u32x4 xv[XQ];
+    };
+    GroupRegs set_a, set_b;
+    // activations first (small, they gate the LDS staging), then scales, then the eight packed rows
+    auto issue_loads = [&](int g, GroupRegs& r) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < XQ; ++i) {
             const int m = i * 4 + kq;
-            xv[i] = u32x4{0u, 0u, 0u, 0u};
+            r.xv[i] = u32x4{0u, 0u, 0u, 0u};
             if (m < a.M && (!EXT || 128 * g + 8 * slot < a.k_valid))
-                xv[i] = *reinterpret_cast<const u32x4*>(a.X + (size_t)m * a.ldx + 128 * g + 8 * slot);
+                r.xv[i] = *reinterpret_cast<const u32x4*>(a.X + (size_t)m * a.ldx + 128 * g + 8 * slot);
         }
         if (!a.per_column) {
-            sc = *reinterpret_cast<const u32x4*>(strip_s + (size_t)g * a.N + scale_off);
+            r.sc = *reinterpret_cast<const u32x4*>(strip_s + (size_t)g * a.N + scale_off);
         } else {
             uint32_t t[4];
 #pragma unroll
@@ -140,21 +143,20 @@ void w4a16_stream_kernel(const StreamArgs a) {
                 const uint16_t hi = *reinterpret_cast<const uint16_t*>(a.S + single_scale_pos(n1));
                 t[p] = (uint32_t)lo | ((uint32_t)hi << 16);
             }
-            sc = u32x4{t[0], t[1], t[2], t[3]};
+            r.sc = u32x4{t[0], t[1], t[2], t[3]};
         }
         const u32x4* rowp = strip_w + (size_t)(8 * g) * N4;  // uniform
 #pragma unroll
-        for (int rr = 0; rr < 2 * RPW; ++rr) wq[rr] = __builtin_nontemporal_load(rowp + (size_t)rr * N4 + piece_off);
+        for (int rr = 0; rr < 2 * RPW; ++rr) r.wq[rr] = __builtin_nontemporal_load(rowp + (size_t)rr * N4 + piece_off);
     };
 
-    for (int g = g_begin; g < g_end; ++g) {  // wave-uniform trip count
-        issue_loads(g);
+    auto process = [&](const GroupRegs& r) __attribute__((always_inline)) {
         // ---- rotate (optionally) and stage the activations in LDS ------------------
 #pragma unroll
         for (int i = 0; i < XQ; ++i) {
             const int mrow = i * 4;
             if (mrow < a.xrows) {  // uniform
-                u32x4 v = xv[i];
+                u32x4 v = r.xv[i];
                 if (HAD) {
                     float f[8];
 #pragma unroll
@@ -183,8 +185,6 @@ void w4a16_stream_kernel(const StreamArgs a) {
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        const u32x4 (&cur)[2 * RPW] = wq;
-        const u32x4 sc_cur = sc;
         // Row pair rp (packed rows 2rp, 2rp+1 = 32 K values) against the eight column slots
         // jb = 2j + blk of this lane: the B operand is the four code pairs of words j of both
         // packed rows (low byte pair for blk 0, after >> 8 for blk 1), expanded and scaled; the
@@ -195,8 +195,8 @@ void w4a16_stream_kernel(const StreamArgs a) {
             const h8 xa = __builtin_bit_cast(h8, *reinterpret_cast<const u32x4*>(xs + xrow_of + 16 * rp));
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const uint32_t q0 = cur[2 * rp][j], q1 = cur[2 * rp + 1][j];
-                const h2 pr = bits_to_h2(sc_cur[j]);
+                const uint32_t q0 = r.wq[2 * rp][j], q1 = r.wq[2 * rp + 1][j];
+                const h2 pr = bits_to_h2(r.sc[j]);
 #pragma unroll
                 for (int blk = 0; blk < 2; ++blk) {
                     const uint32_t p0 = blk ? (q0 >> 8) : q0;
@@ -208,6 +208,33 @@ void w4a16_stream_kernel(const StreamArgs a) {
                     acc[2 * j + blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, bw, acc[2 * j + blk], 0, 0, 0);
                 }
             }
+        }
+        // the next group's staging must not overtake this group's operand reads
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    };
+
+    // Wave-uniform trip counts throughout.  Every process() call sits on a path with a fixed
+    // sequence of loads before it, so that the wait the compiler places ahead of the first use
+    // of a set leaves exactly the other set's loads outstanding (a process() reached both with
+    // and without a prefetch behind it would have to wait for everything).
+    if (g_begin < g_end) {
+        int g = g_begin;
+        issue_loads(g, set_a);
+        while (g + 2 < g_end) {
+            issue_loads(g + 1, set_b);
+            process(set_a);
+            issue_loads(g + 2, set_a);
+            process(set_b);
+            g += 2;
+        }
+        if (g + 1 < g_end) {
+            issue_loads(g + 1, set_b);
+            process(set_a);
+            process(set_b);
+        } else {
+            process(set_a);
         }
     }
 
@@ -420,6 +447,87 @@ int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const 
         if (e != hipSuccess) return UNIQL_E_LAUNCH;
     }
     return UNIQL_OK;
+}
+
+// ---------------------------------------------------------------------------------
+// Measurement aid: what the memory system alone allows for a streaming launch.  Same grid,
+// same wave count, same strip / split / group walk and the same 16-byte nontemporal loads of
+// packed rows and scales as w4a16_stream_kernel, but the data is only XOR-ed together (36
+// instructions per unit) and nothing is staged, expanded, multiplied, reduced or exchanged;
+// one dword per wave is stored if the XOR hits a value that random data practically never
+// produces, so the loads cannot be dropped.  DEPTH units are requested before the first is
+// consumed.
+template <int WAVES, int DEPTH>
+__global__ __launch_bounds__(64 * WAVES, 2)
+void w4a16_read_floor_kernel(const u32x4* B, const half_t* S, int N, int G, int upw, uint32_t* sink) {
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int slot = lane & 15, kq = lane >> 4, c8 = slot & 7;
+    const int nstrips = N >> 7;
+    const int strip = blockIdx.x % nstrips;
+    const int split = blockIdx.x / nstrips;
+    const int N4 = N >> 1;
+    const int g_begin = (split * WAVES + w) * upw;
+    const int g_end = (g_begin + upw < G) ? (g_begin + upw) : G;
+    const uint32_t piece_off = (uint32_t)((slot >> 3) * 32 + 4 * c8 + kq);
+    const uint32_t scale_off = (uint32_t)((slot >> 3) * 64 + 8 * c8);
+    const u32x4* strip_w = B + (size_t)strip * 64;
+    const half_t* strip_s = S + (size_t)strip * 128;
+    u32x4 x = u32x4{0u, 0u, 0u, 0u};
+    for (int g0 = g_begin; g0 < g_end; g0 += DEPTH) {
+        u32x4 wq[DEPTH][8], sc[DEPTH];
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            const int g = g0 + d < g_end ? g0 + d : g_end - 1;  // past the end: the last unit again (depth > 1 only)
+            sc[d] = *reinterpret_cast<const u32x4*>(strip_s + (size_t)g * N + scale_off);
+            const u32x4* rowp = strip_w + (size_t)(8 * g) * N4;
+#pragma unroll
+            for (int rr = 0; rr < 8; ++rr) wq[d][rr] = __builtin_nontemporal_load(rowp + (size_t)rr * N4 + piece_off);
+        }
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            x ^= sc[d];
+#pragma unroll
+            for (int rr = 0; rr < 8; ++rr) x ^= wq[d][rr];
+        }
+    }
+    if ((x[0] ^ x[1] ^ x[2] ^ x[3]) == 0x9e3779b9u) sink[blockIdx.x * WAVES + w] = x[0];
+}
+
+template <int WAVES>
+static void read_floor_depth(int depth, int grid, hipStream_t stream, const u32x4* B, const half_t* S, int N, int G,
+                             int upw, uint32_t* sink) {
+    if (depth >= 4)
+        hipLaunchKernelGGL((w4a16_read_floor_kernel<WAVES, 4>), dim3(grid), dim3(64 * WAVES), 0, stream, B, S, N, G, upw, sink);
+    else if (depth >= 2)
+        hipLaunchKernelGGL((w4a16_read_floor_kernel<WAVES, 2>), dim3(grid), dim3(64 * WAVES), 0, stream, B, S, N, G, upw, sink);
+    else
+        hipLaunchKernelGGL((w4a16_read_floor_kernel<WAVES, 1>), dim3(grid), dim3(64 * WAVES), 0, stream, B, S, N, G, upw, sink);
+}
+
+// tune: as stream_launch (bits 0..7 groups per wave, bits 8..12 waves per workgroup), plus bits
+// 13..15 the number of units a wave requests before it consumes the first (0 = 1)
+int read_floor_launch(const void* B, const void* S, void* sink, int m, int n, int k, unsigned tune, hipStream_t stream) {
+    int waves_override = (int)((tune >> 8) & 0x1fu);
+    if (waves_override != 4 && waves_override != 8) waves_override = 0;
+    const StreamPlan plan = stream_plan(m < 16 ? m : 16, n, k, (int)(tune & 0xffu), waves_override);
+    const int depth = (int)((tune >> 13) & 7u);
+    const int grid = (n / 128) * plan.splits;
+    if (plan.waves == 8)
+        read_floor_depth<8>(depth, grid, stream, reinterpret_cast<const u32x4*>(B), reinterpret_cast<const half_t*>(S), n,
+                            k / 128, plan.upw, reinterpret_cast<uint32_t*>(sink));
+    else
+        read_floor_depth<4>(depth, grid, stream, reinterpret_cast<const u32x4*>(B), reinterpret_cast<const half_t*>(S), n,
+                            k / 128, plan.upw, reinterpret_cast<uint32_t*>(sink));
+    return hipGetLastError() == hipSuccess ? UNIQL_OK : UNIQL_E_LAUNCH;
+}
+
+size_t read_floor_sink_bytes(int m, int n, int k, unsigned tune) {
+    int waves_override = (int)((tune >> 8) & 0x1fu);
+    if (waves_override != 4 && waves_override != 8) waves_override = 0;
+    const StreamPlan plan = stream_plan(m < 16 ? m : 16, n, k, (int)(tune & 0xffu), waves_override);
+    return (size_t)(n / 128) * plan.splits * plan.waves * sizeof(uint32_t);
 }
 
 }  // namespace uniql

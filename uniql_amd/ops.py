@@ -21,7 +21,7 @@ from . import _capi
 __all__ = [
     "w4a16o16_gemm", "w4a16_gemm_ex", "w4a16_linear", "w4a16_dequant", "w4a16_embedding_lookup",
     "fast_hadamard_transform", "hadamard_blockwise", "unsupported_hadamard_variant",
-    "w4a16_quantize", "w4a16_pack", "w4a16_unpack", "w4_embedding_quantize", "rope_indices_",
+    "w4a16_read_floor", "w4a16_quantize", "w4a16_pack", "w4a16_unpack", "w4_embedding_quantize", "rope_indices_",
 ]
 
 
@@ -272,6 +272,25 @@ def w4a16_dequant(B: torch.Tensor, s: torch.Tensor, size_n: int, size_k: int, wa
                                        size_n, size_k, s.shape[0], _stream_ptr(dev))
     _capi.check(code, "uniql_w4a16_dequant")
     return (W, codes) if want_codes else W
+
+
+def w4a16_read_floor(B: torch.Tensor, s: torch.Tensor, size_m: int, size_n: int, size_k: int, flags: int = 0) -> None:
+    """Measurement aid: enqueues the kernel that only reads what the streaming kernel reads for
+    this shape (uniql_w4a16_read_floor), with the same plan.  Returns nothing."""
+    _require_gpu(B, "B")
+    _require_gpu(s, "s")
+    if B.dtype != torch.int32 or s.dtype != torch.float16 or not (B.is_contiguous() and s.is_contiguous()):
+        raise RuntimeError("B must be contiguous int32 and s contiguous float16")
+    if tuple(B.shape) != (size_k // 16, 2 * size_n) or tuple(s.shape) != (size_k // 128, size_n):
+        raise RuntimeError("B / s shapes do not match size_k, size_n (group-128 scales)")
+    lib = _capi.load()
+    dev = B.device
+    with _device_guard(dev):
+        need = lib.uniql_w4a16_read_floor_sink_bytes(size_m, size_n, size_k, flags)
+        sink = torch.empty(max(need, 4), dtype=torch.uint8, device=dev)
+        code = lib.uniql_w4a16_read_floor(B.data_ptr(), s.data_ptr(), sink.data_ptr(), sink.numel(), size_m, size_n,
+                                          size_k, flags, _stream_ptr(dev))
+    _capi.check(code, "uniql_w4a16_read_floor")
 
 
 def w4a16_quantize(weight: torch.Tensor, given_scale: torch.Tensor | None = None, pad_out: int = 0):
