@@ -29,7 +29,8 @@ enum {
     UNIQL_E_ALIGN = -3,       /* a pointer or leading dimension is not 16-byte aligned */
     UNIQL_E_WORKSPACE = -4,   /* workspace, accum or temp buffer too small         */
     UNIQL_E_UNSUPPORTED = -5, /* valid request this build does not implement       */
-    UNIQL_E_LAUNCH = -6       /* the HIP runtime rejected a launch                 */
+    UNIQL_E_LAUNCH = -6,      /* the HIP runtime rejected a launch                 */
+    UNIQL_E_STATIC_LIMIT = -7 /* uniql_w4a16_gemm_static: the call needs more scratch than the static buffer holds */
 };
 
 /* flags of uniql_w4a16_gemm */
@@ -113,6 +114,29 @@ int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, v
                      int m, int n, int k, int groups,
                      int had_block, float had_scale,
                      unsigned flags, void* stream);
+
+/*
+ * uniql_w4a16_gemm for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose
+ * wrapper allocates its reduction buffer on every call (csrc/linear/marlin_gemm_kernel.cuh:1018).
+ * Same arguments and results as uniql_w4a16_gemm without `accum` and `temp`: both come from a
+ * 16 MiB array inside the library's device image (one copy per GPU, held until the process ends):
+ * uniql_w4a16_gemm_static_limit(0) bytes of exchange words (4 MiB: the streaming kernel's 16-row
+ * slab up to n = 32768) and uniql_w4a16_gemm_static_limit(1) bytes of temporary area (12 MiB:
+ * rotated activations, the tiled kernel's partial tiles).  A call whose plan needs more of either
+ * (uniql_w4a16_linear_workspace tells) returns UNIQL_E_STATIC_LIMIT and launches nothing.  The
+ * call itself allocates and frees nothing; it enqueues one small clearing kernel for the
+ * exchange words it will use, then the kernels of uniql_w4a16_gemm.
+ * Every call on a GPU shares that GPU's array: calls that may overlap on one GPU (different
+ * streams, or graphs replayed concurrently) race and must use uniql_w4a16_gemm with separate
+ * buffers instead.
+ */
+size_t uniql_w4a16_gemm_static_limit(int which);
+int uniql_w4a16_gemm_static(const void* A, int64_t lda, const void* B, const void* S, void* D,
+                            const int32_t* workspace, int64_t workspace_len,
+                            int m, int n, int k, int groups,
+                            int had_block, float had_scale,
+                            unsigned flags, void* stream);
 
 /*
  * The whole forward of the reference's layer in one call, with the work around the product

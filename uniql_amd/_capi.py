@@ -29,6 +29,9 @@ SIGNATURES = {
     "uniql_w4a16_gemm": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
                                  c_void_p, c_int64, c_void_p, c_size_t, c_void_p, c_size_t,
                                  c_int, c_int, c_int, c_int, c_int, c_float, c_uint, c_void_p]),
+    "uniql_w4a16_gemm_static_limit": (c_size_t, [c_int]),
+    "uniql_w4a16_gemm_static": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
+                                        c_int, c_int, c_int, c_int, c_int, c_float, c_uint, c_void_p]),
     "uniql_w4a16_linear_temp_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "uniql_w4a16_linear_workspace": (c_int, [c_int, c_int, c_int, c_int, c_int, c_uint,
                                              ctypes.POINTER(c_size_t), ctypes.POINTER(c_size_t)]),

@@ -1,5 +1,7 @@
 // extern "C" surface: argument checks and dispatch.  Nothing here allocates,
 // synchronises or throws.
+#include <mutex>
+
 #include "common.hpp"
 
 namespace uniql {
@@ -69,6 +71,9 @@ const char* uniql_status_string(int code) {
         case UNIQL_E_WORKSPACE: return "workspace, accum or temp buffer too small";
         case UNIQL_E_UNSUPPORTED: return "request not supported by this build";
         case UNIQL_E_LAUNCH: return "HIP runtime rejected the kernel launch";
+        case UNIQL_E_STATIC_LIMIT:
+            return "the call needs more scratch memory than the library's static buffer holds "
+                   "(uniql_w4a16_gemm_static_limit); use uniql_w4a16_gemm with caller-provided buffers";
         default: return "unknown status";
     }
 }
@@ -129,11 +134,13 @@ size_t uniql_w4a16_gemm_temp_bytes(int m, int n, int k, int had_block) {
     return uniql_w4a16_linear_temp_bytes(m, n, k, k, had_block);
 }
 
-int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, const void* S, const void* bias,
+// check_only: every argument check, then return before the first kernel is enqueued
+static int linear_impl(const void* A, int64_t lda, int k_in, const void* B, const void* S, const void* bias,
                        const void* residual, int64_t ldr, void* D, int64_t ldd, int n_out, int epilogue,
                        const int32_t* workspace,
                        int64_t workspace_len, void* accum, size_t accum_bytes, void* temp, size_t temp_bytes, int m,
-                       int n, int k, int groups, int had_block, float had_scale, unsigned flags, void* stream) {
+                       int n, int k, int groups, int had_block, float had_scale, unsigned flags, void* stream,
+                       bool check_only) {
     const int rc = check_linear_shape(m, n, k, groups);
     if (rc != UNIQL_OK) return rc;
     const bool transpose = (flags & UNIQL_F_TRANSPOSE_OUT) != 0;
@@ -179,6 +186,7 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
     void* part = part_bytes ? reinterpret_cast<char*>(temp) + act_bytes : nullptr;
     // last check before the first kernel is enqueued: whether the tiled kernel can take the shape
     if (!use_stream && !tile_shape_ok(m, n, k, (rotate_first || pad_first) ? (int64_t)k : lda, tune)) return UNIQL_E_SHAPE;
+    if (check_only) return UNIQL_OK;
     if (pad_first) {
         const int e = pad_rows_launch(A, lda, k_in, temp, k, m, st);
         if (e != UNIQL_OK) return e;
@@ -208,15 +216,99 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
     return tile_launch(Ain, ld, B, S, D, epi, accum, accum_bytes, part, part_bytes, m, n, k, groups, tune, st);
 }
 
-int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, void* D, const int32_t* workspace,
+int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, const void* S, const void* bias,
+                       const void* residual, int64_t ldr, void* D, int64_t ldd, int n_out, int epilogue,
+                       const int32_t* workspace,
+                       int64_t workspace_len, void* accum, size_t accum_bytes, void* temp, size_t temp_bytes, int m,
+                       int n, int k, int groups, int had_block, float had_scale, unsigned flags, void* stream) {
+    return linear_impl(A, lda, k_in, B, S, bias, residual, ldr, D, ldd, n_out, epilogue, workspace, workspace_len, accum,
+                       accum_bytes, temp, temp_bytes, m, n, k, groups, had_block, had_scale, flags, stream, false);
+}
+
+static int gemm_impl(const void* A, int64_t lda, const void* B, const void* S, void* D, const int32_t* workspace,
                      int64_t workspace_len, void* accum, size_t accum_bytes, void* temp, size_t temp_bytes, int m,
-                     int n, int k, int groups, int had_block, float had_scale, unsigned flags, void* stream) {
+                     int n, int k, int groups, int had_block, float had_scale, unsigned flags, void* stream,
+                     bool check_only) {
     if (D && !aligned16(D)) return UNIQL_E_ALIGN;
     // transposed: D is [n, m8] with m8 = m rounded up to 8, as the reference allocates it
     // (marlin_gemm_kernel.cuh:1023-1026)
     const int64_t ldd = (flags & UNIQL_F_TRANSPOSE_OUT) ? (int64_t)((m + 7) / 8) * 8 : n;
-    return uniql_w4a16_linear(A, lda, k, B, S, nullptr, nullptr, 0, D, ldd, n, UNIQL_EPI_NONE, workspace, workspace_len, accum,
-                              accum_bytes, temp, temp_bytes, m, n, k, groups, had_block, had_scale, flags, stream);
+    return linear_impl(A, lda, k, B, S, nullptr, nullptr, 0, D, ldd, n, UNIQL_EPI_NONE, workspace, workspace_len, accum,
+                       accum_bytes, temp, temp_bytes, m, n, k, groups, had_block, had_scale, flags, stream, check_only);
+}
+
+int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, void* D, const int32_t* workspace,
+                     int64_t workspace_len, void* accum, size_t accum_bytes, void* temp, size_t temp_bytes, int m,
+                     int n, int k, int groups, int had_block, float had_scale, unsigned flags, void* stream) {
+    return gemm_impl(A, lda, B, S, D, workspace, workspace_len, accum, accum_bytes, temp, temp_bytes, m, n, k, groups,
+                     had_block, had_scale, flags, stream, false);
+}
+
+// ---- the entry point that allocates nothing --------------------------------------------------
+// All the scratch memory a product needs (the zero-in / zero-out exchange words first, then the
+// temporary area) lives in one array in this library's device image.  Each GPU holds its own copy
+// at its own address; the name below is only a host-side handle for hipGetSymbolAddress, never a
+// device address, so every use goes through the per-device pointer looked up once.
+static constexpr size_t kStaticAccumBytes = (size_t)4 << 20;   // exchange words: 16 rows x 32768 columns
+static constexpr size_t kStaticTempBytes = (size_t)12 << 20;   // rotated rows / partial tiles
+static __device__ __align__(256) unsigned char scratch[kStaticAccumBytes + kStaticTempBytes];
+
+static constexpr int kMaxDevices = 64;
+static std::mutex g_scratch_mutex;
+static unsigned char* g_scratch_ptr[kMaxDevices];  // zero-initialised: not looked up yet
+
+// the current device's copy of the array, or nullptr
+static unsigned char* static_scratch() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return nullptr;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)) != hipSuccess) return nullptr;
+        g_scratch_ptr[dev] = reinterpret_cast<unsigned char*>(p);
+    }
+    return g_scratch_ptr[dev];
+}
+
+__global__ __launch_bounds__(256) void clear_words_kernel(u32x4* p, size_t count) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < count) p[i] = u32x4{0u, 0u, 0u, 0u};
+}
+
+size_t uniql_w4a16_gemm_static_limit(int which) {
+    return which == 0 ? kStaticAccumBytes : (which == 1 ? kStaticTempBytes : 0);
+}
+
+int uniql_w4a16_gemm_static(const void* A, int64_t lda, const void* B, const void* S, void* D,
+                            const int32_t* workspace, int64_t workspace_len, int m, int n, int k, int groups,
+                            int had_block, float had_scale, unsigned flags, void* stream) {
+    const int rc = check_linear_shape(m, n, k, groups);
+    if (rc != UNIQL_OK) return rc;
+    if (m == 0) return UNIQL_OK;
+    size_t need_accum = 0, need_temp = 0;
+    const int wrc = uniql_w4a16_linear_workspace(m, n, k, k, had_block, flags, &need_accum, &need_temp);
+    if (wrc != UNIQL_OK) return wrc;
+    if (need_accum > kStaticAccumBytes || need_temp > kStaticTempBytes) return UNIQL_E_STATIC_LIMIT;
+    if (!A || !B || !S || !D) return UNIQL_E_NULL;
+    unsigned char* base = static_scratch();
+    if (!base) return UNIQL_E_LAUNCH;
+    void* accum = need_accum ? base : nullptr;
+    void* temp = need_temp ? base + kStaticAccumBytes : nullptr;
+    // every argument check of the product first: nothing is enqueued for a call that will be refused
+    const int crc = gemm_impl(A, lda, B, S, D, workspace, workspace_len, accum, need_accum, temp, need_temp, m, n, k,
+                              groups, had_block, had_scale, flags, stream, true);
+    if (crc != UNIQL_OK) return crc;
+    // The exchange words must be zero on entry.  The kernels leave them zero, but the array is
+    // shared by every call on this GPU, so the part this call uses is cleared by a small kernel
+    // (a kernel, not a memset node: the call may be recorded into a graph).
+    if (need_accum > 0) {
+        const size_t count = need_accum / sizeof(u32x4);
+        hipLaunchKernelGGL(clear_words_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0,
+                           reinterpret_cast<hipStream_t>(stream), reinterpret_cast<u32x4*>(base), count);
+        if (hipGetLastError() != hipSuccess) return UNIQL_E_LAUNCH;
+    }
+    return gemm_impl(A, lda, B, S, D, workspace, workspace_len, accum, need_accum, temp, need_temp, m, n, k, groups,
+                     had_block, had_scale, flags, stream, false);
 }
 
 int uniql_w4a16_read_floor(const void* B, const void* S, void* sink, size_t sink_bytes, int m, int n, int k,

@@ -19,7 +19,7 @@ import torch
 from . import _capi
 
 __all__ = [
-    "w4a16o16_gemm", "w4a16_gemm_ex", "w4a16_linear", "w4a16_dequant", "w4a16_embedding_lookup",
+    "w4a16o16_gemm", "w4a16_gemm_ex", "w4a16_gemm_static", "w4a16_linear", "w4a16_dequant", "w4a16_embedding_lookup",
     "fast_hadamard_transform", "hadamard_blockwise", "unsupported_hadamard_variant",
     "w4a16_read_floor", "w4a16_quantize", "w4a16_pack", "w4a16_unpack", "w4_embedding_quantize", "rope_indices_",
 ]
@@ -159,6 +159,37 @@ def w4a16_gemm_ex(A: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: 
             size_m, size_n, size_k, groups, had_block, float(had_scale), flags, _stream_ptr(dev))
     _capi.check(code, "uniql_w4a16_gemm")
     return D
+
+
+def w4a16_gemm_static(A: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: torch.Tensor, out: torch.Tensor,
+                      size_m: int, size_n: int, size_k: int, *, had_block: int = 0, had_scale: float = 1.0,
+                      flags: int = 0) -> torch.Tensor:
+    """uniql_w4a16_gemm_static: the product into the caller's `out` with the library's own static
+    scratch memory; neither this wrapper nor the call allocates anything.  Raises when the call's
+    plan needs more scratch than the static buffer holds."""
+    for t, name in ((A, "A"), (B, "B"), (s, "s"), (workspace, "workspace"), (out, "out")):
+        _require_gpu(t, name)
+    if A.dtype != torch.float16 or s.dtype != torch.float16 or B.dtype != torch.int32 or workspace.dtype != torch.int32:
+        raise RuntimeError("A and s must be float16, B and workspace int32")
+    want = torch.float32 if flags & _capi.F_OUT_F32 else torch.float16
+    if out.dtype != want or not out.is_contiguous() or tuple(out.shape) != (size_m, size_n):
+        raise RuntimeError(f"out must be a contiguous {want} tensor of shape ({size_m}, {size_n})")
+    if flags & _capi.F_TRANSPOSE_OUT:
+        raise RuntimeError("transposed output is not offered by this wrapper")
+    if A.dim() != 2 or A.stride(1) != 1 or tuple(A.shape) != (size_m, size_k):
+        raise RuntimeError(f"A must be ({size_m}, {size_k}) with unit stride along K")
+    if not (B.is_contiguous() and s.is_contiguous()) or tuple(B.shape) != (size_k // 16, 2 * size_n) or \
+            s.dim() != 2 or s.shape[1] != size_n:
+        raise RuntimeError("B / s shapes do not match size_k, size_n")
+    lib = _capi.load()
+    dev = A.device
+    with _device_guard(dev):
+        code = lib.uniql_w4a16_gemm_static(
+            A.data_ptr(), A.stride(0) if size_m > 1 else size_k, B.data_ptr(), s.data_ptr(), out.data_ptr(),
+            workspace.data_ptr(), workspace.numel(), size_m, size_n, size_k, s.shape[0], had_block,
+            float(had_scale), flags, _stream_ptr(dev))
+    _capi.check(code, "uniql_w4a16_gemm_static")
+    return out
 
 
 def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: torch.Tensor, size_n: int,
