@@ -88,6 +88,7 @@ class Layer:
         return ops.w4a16o16_gemm(self.x, b, s, self.ws, self.m, self.n, self.k, False, -1, -1, -1, 16)
 
 
+SETTLE_MS = 10.0   # untimed replays before every timed region, whatever --warmup says
 GRAPH_STEPS = 40   # steps captured per HIP graph (a decode step of a 32-layer model replays more kernels than that)
 
 
@@ -116,10 +117,18 @@ def time_graphs(run_step, n_variants, steps, warmup):
     per_graph = n_variants * max(1, min(steps, GRAPH_STEPS) // n_variants)
     full = capture(per_graph)
     rest = capture(steps % per_graph) if steps % per_graph else None
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    # untimed: the `warmup` steps asked for, and in any case SETTLE_MS of replays, because the clocks of a
+    # chip that was idle need several milliseconds of load to settle (one replay is well under 1 ms)
+    start.record()
     for _ in range(max(1, warmup // per_graph)):
         full.replay()
+    stop.record()
     torch.cuda.synchronize()
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    per_replay_ms = max(start.elapsed_time(stop) / max(1, warmup // per_graph), 1e-3)
+    for _ in range(int(SETTLE_MS / per_replay_ms) + 1):
+        full.replay()
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
     start.record()
     for _ in range(steps // per_graph):

@@ -329,24 +329,26 @@ struct StreamPlan {
     int splits;
 };
 
-// Heuristic (from sweeps over waves x groups per wave on the Llama shapes):
-//   * enough strips to occupy the chip on their own (>= 192): one workgroup of 8 waves owns a
-//     whole strip, so no partial sums are exchanged between workgroups;
-//   * otherwise K is split over workgroups.  One or two rows: 4 waves (8 when that still leaves
-//     fewer than three waves per SIMD), about 1024 workgroups at most.  More rows: every split
-//     costs a 64-bit atomic per output element, so 8 waves and at most about 256 workgroups.
+// Heuristic (from sweeps over waves x groups per wave on the Llama, pruned-Llama and Mamba2 shapes
+// at 1, 2, 4 and 8 rows):
+//   * enough strips to occupy the chip on their own (>= 176): one workgroup owns a whole strip, so
+//     no partial sums are exchanged between workgroups; four waves with eight groups each when K
+//     allows it (long streams per wave, two register sets in flight), else eight waves;
+//   * otherwise K is split over workgroups.  One or two rows: 4 waves, and as many groups per wave
+//     as it takes to stay within about 288 workgroups.  More rows: every split costs a 64-bit
+//     atomic per output element, so 8 waves (4 for small problems) and at most 256 workgroups.
 static StreamPlan stream_plan(int m, int n, int k, int upw_override, int waves_override) {
     const int nstrips = n / 128, G = k / 128;
     const int64_t units = (int64_t)nstrips * G;
     StreamPlan p;
-    const bool whole_strip = m <= 16 && nstrips >= 192 && G >= 16 && G <= 64;
-    int max_wgs = 1024;
+    const bool whole_strip = m <= 16 && nstrips >= 176 && G >= 16 && G <= 64;
+    int max_wgs = 288;
     if (waves_override) {
         p.waves = waves_override;
     } else if (whole_strip) {
-        p.waves = 8;
+        p.waves = G <= 32 ? 4 : 8;
     } else if (m <= 2) {
-        p.waves = (units >= 1536 && units < 3072) ? 8 : 4;
+        p.waves = 4;
     } else {
         p.waves = (m <= 16 && units >= 1536) ? 8 : 4;
         max_wgs = 256;
@@ -357,7 +359,7 @@ static StreamPlan stream_plan(int m, int n, int k, int upw_override, int waves_o
         p.upw = ceil_div(G, p.waves);
     } else {
         p.upw = 1;
-        while (p.upw < 8 && (int64_t)nstrips * ceil_div(G, p.waves * p.upw) > max_wgs) p.upw *= 2;
+        while (p.upw < 8 && (int64_t)nstrips * ceil_div(G, p.waves * p.upw) > max_wgs) ++p.upw;
     }
     p.splits = ceil_div(G, p.waves * p.upw);
     while (p.splits > kAccumMaxSplits) {  // the contribution count has 7 bits
