@@ -9,6 +9,7 @@ int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const 
                   const Epilogue& epi, void* accum, int m, int n, int k, int groups, bool had128, float had_scale,
                   unsigned tune, hipStream_t stream);
 size_t stream_accum_bytes(int m, int n, int k);
+bool stream_shape_ok(int k, int64_t lda);
 int read_floor_launch(const void* B, const void* S, void* sink, int m, int n, int k, unsigned tune, hipStream_t stream);
 size_t read_floor_sink_bytes(int m, int n, int k, unsigned tune);
 int tile_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, const Epilogue& epi, void* accum,
@@ -186,6 +187,7 @@ static int linear_impl(const void* A, int64_t lda, int k_in, const void* B, cons
     void* part = part_bytes ? reinterpret_cast<char*>(temp) + act_bytes : nullptr;
     // last check before the first kernel is enqueued: whether the tiled kernel can take the shape
     if (!use_stream && !tile_shape_ok(m, n, k, (rotate_first || pad_first) ? (int64_t)k : lda, tune)) return UNIQL_E_SHAPE;
+    if (use_stream && !stream_shape_ok(k, (rotate_first || pad_first) ? (int64_t)k : lda)) return UNIQL_E_SHAPE;
     if (check_only) return UNIQL_OK;
     if (pad_first) {
         const int e = pad_rows_launch(A, lda, k_in, temp, k, m, st);

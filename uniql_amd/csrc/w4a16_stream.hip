@@ -55,6 +55,7 @@ struct StreamArgs {
     int splits;           // workgroups along K per strip
     int xrows;            // activation rows staged per wave: M rounded up to a multiple of 4
     int k_valid;          // columns of X that exist (multiple of 8); the rest of K counts as zeros
+    unsigned x_bytes;     // bytes from X to the end of its last row (< 2 GiB: buffer addressing)
     float had_scale;
     Epilogue epi;
 };
@@ -84,9 +85,8 @@ void w4a16_stream_kernel(const StreamArgs a) {
     const int kq = lane >> 4;
     const int c8 = slot & 7;
 
-    const int nstrips = a.N >> 7;
-    const int strip = blockIdx.x % nstrips;
-    const int split = blockIdx.x / nstrips;
+    const int strip = blockIdx.x;
+    const int split = blockIdx.y;
 
     const int N4 = a.N >> 1;  // 16-byte pieces per packed row
     const int g_begin = (split * WAVES + w) * a.upw;
@@ -123,34 +123,36 @@ void w4a16_stream_kernel(const StreamArgs a) {
         u32x4 xv[XQ];
     };
     GroupRegs set_a, set_b;
+    // Activation rows are read through a buffer descriptor: a lane whose row does not exist (or,
+    // with a short input, whose columns do not) uses an offset beyond the descriptor and gets zeros.
+    // No branch around a load: the code from the kernel's entry to the first group's loads is one
+    // block, so the kernel arguments are fetched together and the loads leave as early as possible.
+    const __amdgpu_buffer_rsrc_t x_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(a.X), 0, a.x_bytes, 0x00020000);
+    uint32_t x_off[XQ];
+#pragma unroll
+    for (int i = 0; i < XQ; ++i) {
+        const int m = 4 * i + kq;
+        x_off[i] = m < a.M ? (uint32_t)m * (uint32_t)a.ldx * 2u + 16u * (uint32_t)slot : 0x80000000u;
+    }
     // activations first (small, they gate the LDS staging), then scales, then the eight packed rows
     auto issue_loads = [&](int g, GroupRegs& r) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < XQ; ++i) {
-            const int m = i * 4 + kq;
-            r.xv[i] = u32x4{0u, 0u, 0u, 0u};
-            if (m < a.M && (!EXT || 128 * g + 8 * slot < a.k_valid))
-                r.xv[i] = *reinterpret_cast<const u32x4*>(a.X + (size_t)m * a.ldx + 128 * g + 8 * slot);
+            uint32_t off = x_off[i];
+            if (EXT) off = 128 * g + 8 * slot < a.k_valid ? off : 0x80000000u;
+            r.xv[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, off, 256u * (uint32_t)g, 0));
         }
-        if (!a.per_column) {
-            r.sc = *reinterpret_cast<const u32x4*>(strip_s + (size_t)g * a.N + scale_off);
-        } else {
-            uint32_t t[4];
-#pragma unroll
-            for (int p = 0; p < 4; ++p) {
-                const int n0 = strip * 128 + (slot >> 3) * 64 + c8 + 8 * (2 * p), n1 = n0 + 8;
-                const uint16_t lo = *reinterpret_cast<const uint16_t*>(a.S + single_scale_pos(n0));
-                const uint16_t hi = *reinterpret_cast<const uint16_t*>(a.S + single_scale_pos(n1));
-                t[p] = (uint32_t)lo | ((uint32_t)hi << 16);
-            }
-            r.sc = u32x4{t[0], t[1], t[2], t[3]};
-        }
+        // (one scale row: the load of row 0 is not used, see sc_fixed)
+        r.sc = *reinterpret_cast<const u32x4*>(strip_s + (size_t)(a.per_column ? 0 : g) * a.N + scale_off);
         const u32x4* rowp = strip_w + (size_t)(8 * g) * N4;  // uniform
 #pragma unroll
         for (int rr = 0; rr < 2 * RPW; ++rr) r.wq[rr] = __builtin_nontemporal_load(rowp + (size_t)rr * N4 + piece_off);
     };
 
+    u32x4 sc_fixed = u32x4{0u, 0u, 0u, 0u};  // one scale per column: the same eight scales for every group
     auto process = [&](const GroupRegs& r) __attribute__((always_inline)) {
+        const u32x4 scales = a.per_column ? sc_fixed : r.sc;
         // ---- rotate (optionally) and stage the activations in LDS ------------------
 #pragma unroll
         for (int i = 0; i < XQ; ++i) {
@@ -196,7 +198,7 @@ void w4a16_stream_kernel(const StreamArgs a) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const uint32_t q0 = r.wq[2 * rp][j], q1 = r.wq[2 * rp + 1][j];
-                const h2 pr = bits_to_h2(r.sc[j]);
+                const h2 pr = bits_to_h2(scales[j]);
 #pragma unroll
                 for (int blk = 0; blk < 2; ++blk) {
                     const uint32_t p0 = blk ? (q0 >> 8) : q0;
@@ -219,9 +221,22 @@ void w4a16_stream_kernel(const StreamArgs a) {
     // sequence of loads before it, so that the wait the compiler places ahead of the first use
     // of a set leaves exactly the other set's loads outstanding (a process() reached both with
     // and without a prefetch behind it would have to wait for everything).
+    // the first group's loads leave before anything else is decided (a wave without groups asks
+    // for the last group and ignores it)
+    issue_loads(g_begin < a.G ? g_begin : a.G - 1, set_a);
+    if (a.per_column) {  // uniform, rare
+        uint32_t t[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const int n0 = strip * 128 + (slot >> 3) * 64 + c8 + 8 * (2 * p), n1 = n0 + 8;
+            const uint16_t lo = *reinterpret_cast<const uint16_t*>(a.S + single_scale_pos(n0));
+            const uint16_t hi = *reinterpret_cast<const uint16_t*>(a.S + single_scale_pos(n1));
+            t[p] = (uint32_t)lo | ((uint32_t)hi << 16);
+        }
+        sc_fixed = u32x4{t[0], t[1], t[2], t[3]};
+    }
     if (g_begin < g_end) {
         int g = g_begin;
-        issue_loads(g, set_a);
         while (g + 2 < g_end) {
             issue_loads(g + 1, set_b);
             process(set_a);
@@ -390,8 +405,7 @@ static hipError_t launch_one(const StreamArgs& a, hipStream_t stream) {
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
         if (e != hipSuccess) return e;
     }
-    const int grid = (a.N / 128) * a.splits;
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * WAVES), shmem, stream, a);
+    hipLaunchKernelGGL(kern, dim3(a.N / 128, a.splits), dim3(64 * WAVES), shmem, stream, a);
     return hipGetLastError();
 }
 
@@ -417,9 +431,13 @@ static hipError_t launch_rows(const StreamArgs& a, int waves, hipStream_t stream
 // Rows are processed in slabs of at most 16; every slab re-streams the weights.
 // tune: bits 0..7 groups per wave, bits 8..12 waves per workgroup (4 or 8); zero fields mean
 // "choose".
+// the activation rows of a 16-row slab are addressed with 32-bit byte offsets
+bool stream_shape_ok(int k, int64_t lda) { return (15 * lda + k) * 2 < ((int64_t)1 << 31); }
+
 int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const void* S, void* D,
                   const Epilogue& epi, void* accum, int m, int n, int k, int groups, bool had128, float had_scale,
                   unsigned tune, hipStream_t stream) {
+    if (!stream_shape_ok(k, lda)) return UNIQL_E_SHAPE;
     StreamArgs a;
     a.B = reinterpret_cast<const u32x4*>(B);
     a.S = reinterpret_cast<const half_t*>(S);
@@ -441,6 +459,7 @@ int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const 
         a.upw = plan.upw;
         a.splits = plan.splits;
         a.M = mm;
+        a.x_bytes = (unsigned)(((int64_t)(mm - 1) * lda + k_valid) * 2);
         a.xrows = ((mm + 3) / 4) * 4;
         a.X = reinterpret_cast<const half_t*>(A) + (size_t)m0 * lda;
         a.D = reinterpret_cast<char*>(D) + (size_t)m0 * (epi.transpose ? 1 : epi.ldd) * out_elt;
