@@ -38,6 +38,9 @@ enum {
     UNIQL_F_OUT_F32 = 1 << 0,      /* D is float32 [m, n] instead of fp16 (test hook: the value before the final rounding) */
     UNIQL_F_FORCE_SKINNY = 1 << 1, /* use the weight-streaming kernel (default for m <= 16) whatever m is */
     UNIQL_F_FORCE_TILED = 1 << 2,  /* use the tiled MFMA kernel (default for m > 16) whatever m is */
+    UNIQL_F_SEPARATE_ROTATION = 1 << 4, /* run a whole-row rotation as its own transform kernel into `temp` even
+                                      where the streaming kernel could apply it itself (test hook: both ways
+                                      give the same values bit for bit) */
     UNIQL_F_TRANSPOSE_OUT = 1 << 3 /* the reference's output_transpose ("sequence length last",
                                       csrc/linear/marlin_gemm_kernel.cuh:574-606,1023-1026): D is [n, ldd]
                                       with D[j, i] = product[i, j]; uniql_w4a16_gemm uses ldd = m rounded up
@@ -90,10 +93,12 @@ int uniql_stream_capture_id(void* stream, unsigned long long* id);
  *              concurrently need separate buffers.
  *   had_block  0: none.  Otherwise the activations are rotated first,
  *              A <- fp16(A . H_had_block * had_scale) on consecutive
- *              had_block-wide pieces of each row: 128 is fused into the
- *              streaming kernel's prologue (m <= 16); any other power of two
- *              (<= 32768, dividing k), and 128 for larger m, runs the transform
- *              kernel into `temp` first.
+ *              had_block-wide pieces of each row.  Inside the streaming kernel (m <= 16,
+ *              no extra memory traffic): 128, and had_block == k for a power-of-two k
+ *              with min(m, 16) * k <= 16384 (every workgroup transforms the rows into LDS
+ *              while its first weights are on their way).  Any other power of two
+ *              (<= 32768, dividing k), and every rotation for larger m, runs the
+ *              transform kernel into `temp` first.  Same values either way.
  *   k % 128 == 0, n % 128 == 0 (the module pads n to 256).
  *
  * Partial sums that meet in the streaming kernel's `accum` words are rounded to multiples of

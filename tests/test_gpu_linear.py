@@ -287,6 +287,35 @@ def test_full_width_hadamard_prologue(gpu, m):
     check_fp32_result(y32, p, ref, m, x=xr)
 
 
+@pytest.mark.parametrize("m,k,n", [(1, 8192, 4096), (2, 8192, 384), (1, 16384, 256), (4, 4096, 1024), (3, 2048, 640),
+                                   (16, 1024, 256), (7, 256, 128), (2, 512, 4096)])
+def test_full_row_rotation_inside_the_streaming_kernel(gpu, m, k, n):
+    """Whole-row rotation (block = k) applied by every workgroup of the streaming kernel in LDS against the
+    same call with the transform kernel run first into `temp` (UNIQL_F_SEPARATE_ROTATION): same butterfly
+    order, same single fp16 rounding, so the outputs are identical; and against the oracle."""
+    from uniql_amd import ops, _capi
+    p = make_linear_problem(m, k, n, seed=m * 1000 + k)
+    x, b, s = to_gpu(p, gpu)
+    ws = workspace_for(n, gpu)
+    lib = _capi.load()
+    import ctypes
+    acc, tmp = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    assert lib.uniql_w4a16_linear_workspace(m, n, k, k, k, 0, ctypes.byref(acc), ctypes.byref(tmp)) == 0
+    assert tmp.value == 0                                     # nothing goes through temporary memory
+    assert lib.uniql_w4a16_linear_workspace(m, n, k, k, k, _capi.F_SEPARATE_ROTATION, ctypes.byref(acc), ctypes.byref(tmp)) == 0
+    assert tmp.value == (m * k * 2 + 255) // 256 * 256
+    for out_f32 in (True, False):
+        fused = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k, had_block=k, had_scale=k ** -0.5, out_f32=out_f32)
+        apart = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k, had_block=k, had_scale=k ** -0.5, out_f32=out_f32,
+                                  flags=_capi.F_SEPARATE_ROTATION)
+        assert torch.equal(fused, apart)
+    xr = O.fwht(p["x"], k ** -0.5)
+    ref = O.gemm_fp64(xr, O.dequant_codes(p["q"], p["s"]))
+    check_fp32_result(ops.w4a16_gemm_ex(x, b, s, ws, m, n, k, had_block=k, had_scale=k ** -0.5, out_f32=True).cpu().numpy(),
+                      p, ref, m, x=xr)
+    check_layer_output(fused.cpu().numpy(), ref)
+
+
 @pytest.mark.parametrize("m", [1, 5, 16, 40, 130])
 def test_output_transpose(gpu, m):
     """the reference's output_transpose: D[n, m8], row index last, m rounded up to 8"""

@@ -16,6 +16,7 @@ F_OUT_F32 = 1 << 0
 F_FORCE_SKINNY = 1 << 1
 F_FORCE_TILED = 1 << 2
 F_TRANSPOSE_OUT = 1 << 3
+F_SEPARATE_ROTATION = 1 << 4
 DT_F16, DT_BF16, DT_F32 = 0, 1, 2
 EPI_NONE, EPI_SILU_MUL, EPI_RELU2 = 0, 1, 2
 

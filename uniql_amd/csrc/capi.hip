@@ -6,8 +6,9 @@
 
 namespace uniql {
 int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const void* S, void* D,
-                  const Epilogue& epi, void* accum, int m, int n, int k, int groups, bool had128, float had_scale,
+                  const Epilogue& epi, void* accum, int m, int n, int k, int groups, int had_mode, float had_scale,
                   unsigned tune, hipStream_t stream);
+bool stream_rotates_rows(int m, int k);
 size_t stream_accum_bytes(int m, int n, int k);
 bool stream_shape_ok(int k, int64_t lda);
 int read_floor_launch(const void* B, const void* S, void* sink, int m, int n, int k, unsigned tune, hipStream_t stream);
@@ -90,11 +91,21 @@ static bool takes_stream_kernel(int m, unsigned flags) {
     return use_stream;
 }
 
+// How the streaming kernel itself applies a rotation: 1 the 128-block one while staging, 2 whole
+// rows (block = k, a power of two, few rows, input not shorter than k), 0 not at all: then the
+// transform kernel runs first, into `temp`.
+static int fused_rotation(int m, int k, int k_in, int had_block, bool use_stream, unsigned flags) {
+    if (!use_stream || had_block == 0) return 0;
+    if (had_block == 128) return 1;
+    if (flags & UNIQL_F_SEPARATE_ROTATION) return 0;
+    return (had_block == k && k_in == k && stream_rotates_rows(m, k)) ? 2 : 0;
+}
+
 // bytes of the rotated or zero-padded copy of the activations at the start of `temp`: every
-// rotation except the 128-block one fused into the streaming kernel, and padding whenever the
+// rotation that is not fused into the streaming kernel, and padding whenever the
 // kernel cannot guard its own loads (tiled kernel) or a rotation comes first
-static size_t activation_copy_bytes(int m, int k, int k_in, int had_block, bool use_stream) {
-    const bool rotate_first = had_block != 0 && !(had_block == 128 && use_stream);
+static size_t activation_copy_bytes(int m, int k, int k_in, int had_block, bool use_stream, unsigned flags) {
+    const bool rotate_first = had_block != 0 && fused_rotation(m, k, k_in, had_block, use_stream, flags) == 0;
     const bool pad_first = k_in != k && (rotate_first || !use_stream);
     return (rotate_first || pad_first) ? round256((size_t)m * k * sizeof(half_t)) : 0;
 }
@@ -109,9 +120,9 @@ int uniql_w4a16_linear_workspace(int m, int n, int k, int k_in, int had_block, u
     const unsigned tune = flags >> 8;
     *accum_bytes = round256(use_stream ? stream_accum_bytes(m, n, k) : tile_accum_bytes(m, n, k, tune));
     // a strided input ahead of a separate rotation is compacted into the copy as well: count it
-    const size_t act = had_block != 0 && !(had_block == 128 && use_stream)
+    const size_t act = had_block != 0 && fused_rotation(m, k, k_in, had_block, use_stream, flags) == 0
                            ? round256((size_t)m * k * sizeof(half_t))
-                           : activation_copy_bytes(m, k, k_in, had_block, use_stream);
+                           : activation_copy_bytes(m, k, k_in, had_block, use_stream, flags);
     *temp_bytes = act + (use_stream ? 0 : round256(tile_part_bytes(m, n, k, tune)));
     return UNIQL_OK;
 }
@@ -175,8 +186,8 @@ static int linear_impl(const void* A, int64_t lda, int k_in, const void* B, cons
     const void* Ain = A;
     int64_t ld = lda;
     int k_valid = k_in;
-    const bool had128 = (had_block == 128) && use_stream;
-    const bool rotate_first = had_block != 0 && !had128;
+    const int had_mode = fused_rotation(m, k, k_in, had_block, use_stream, flags);
+    const bool rotate_first = had_block != 0 && had_mode == 0;
     // the transform kernel reads dense rows of k values: a strided or short input is first copied
     // (and zero-padded) into the temporary buffer, then rotated there in place
     const bool pad_first = rotate_first ? (k_in != k || lda != k) : (k_in != k && !use_stream);
@@ -214,7 +225,7 @@ static int linear_impl(const void* A, int64_t lda, int k_in, const void* B, cons
     epi.relu2 = epilogue == UNIQL_EPI_RELU2 ? 1 : 0;
     epi.vec_ok = (!transpose && ldd % 8 == 0 && aligned16(D)) ? 1 : 0;
     if (use_stream)
-        return stream_launch(Ain, ld, k_valid, B, S, D, epi, accum, m, n, k, groups, had128, had_scale, tune, st);
+        return stream_launch(Ain, ld, k_valid, B, S, D, epi, accum, m, n, k, groups, had_mode, had_scale, tune, st);
     return tile_launch(Ain, ld, B, S, D, epi, accum, accum_bytes, part, part_bytes, m, n, k, groups, tune, st);
 }
 

@@ -2,6 +2,7 @@
 // Sylvester (natural-order) matrix, applied to consecutive `block`-wide pieces.
 // Butterflies run in fp32, lowest index bit first, one rounding to fp16 at the end.
 #include "common.hpp"
+#include "fwht_device.hpp"
 
 namespace uniql {
 
@@ -95,38 +96,7 @@ __global__ __launch_bounds__(256) void fwht_lds_kernel(const T* __restrict__ x, 
 }
 
 // ---- fp16, power of two >= 256: vector loads, index bits 0..2 in registers, LDS passes of
-// up to four bits, vector stores --------------------------------------------------------
-// The fp32 image in LDS is padded by eight floats per 128: in the first LDS pass (bits 3..6)
-// the lanes of a wave differ in bits 0..2 and 7.., and the padding moves each step of bit 7
-// to another group of eight banks; the later passes walk consecutive addresses anyway.
-__device__ __forceinline__ int fwht_pad(int idx) { return idx + ((idx >> 7) << 3); }
-
-template <int CNT>
-__device__ __forceinline__ void fwht_pass_padded(float* buf, int L, int lo, int tid, int nthreads) {
-    constexpr int E = 1 << CNT;
-    const int tasks = L >> CNT;
-    const int lowmask = (1 << lo) - 1;
-    for (int t = tid; t < tasks; t += nthreads) {
-        const int base = ((t >> lo) << (lo + CNT)) | (t & lowmask);
-        float v[E];
-#pragma unroll
-        for (int i = 0; i < E; ++i) v[i] = buf[fwht_pad(base + (i << lo))];
-#pragma unroll
-        for (int h = 1; h < E; h <<= 1) {
-#pragma unroll
-            for (int i = 0; i < E; ++i) {
-                if ((i & h) == 0) {
-                    const float p = v[i], q = v[i + h];
-                    v[i] = p + q;
-                    v[i + h] = p - q;
-                }
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < E; ++i) buf[fwht_pad(base + (i << lo))] = v[i];
-    }
-}
-
+// up to four bits (fwht_row_to_lds), vector stores ----------------------------------------------
 __global__ __launch_bounds__(1024) void fwht_f16_kernel(const u32x4* __restrict__ x, u32x4* __restrict__ y, int L,
                                                        int log2L, float scale) {
     extern __shared__ __attribute__((aligned(16))) float fbuf[];
@@ -134,49 +104,7 @@ __global__ __launch_bounds__(1024) void fwht_f16_kernel(const u32x4* __restrict_
     const int chunks = L >> 3;
     const u32x4* xp = x + (size_t)blockIdx.x * chunks;
     u32x4* yp = y + (size_t)blockIdx.x * chunks;
-    for (int c = tid; c < chunks; c += nthreads) {
-        const u32x4 v = xp[c];
-        float f[8];
-#pragma unroll
-        for (int p = 0; p < 4; ++p) {
-            const h2 hv = bits_to_h2(v[p]);
-            f[2 * p] = (float)hv.x;
-            f[2 * p + 1] = (float)hv.y;
-        }
-#pragma unroll
-        for (int h = 1; h < 8; h <<= 1) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                if ((i & h) == 0) {
-                    const float p = f[i], q = f[i + h];
-                    f[i] = p + q;
-                    f[i + h] = p - q;
-                }
-            }
-        }
-        float* dst = fbuf + fwht_pad(8 * c);
-        *reinterpret_cast<f4*>(dst) = f4{f[0], f[1], f[2], f[3]};
-        *reinterpret_cast<f4*>(dst + 4) = f4{f[4], f[5], f[6], f[7]};
-    }
-    __syncthreads();
-    int lo = 3;
-    while (lo < log2L) {
-        const int left = log2L - lo;
-        if (left >= 4) {
-            fwht_pass_padded<4>(fbuf, L, lo, tid, nthreads);
-            lo += 4;
-        } else if (left == 3) {
-            fwht_pass_padded<3>(fbuf, L, lo, tid, nthreads);
-            lo += 3;
-        } else if (left == 2) {
-            fwht_pass_padded<2>(fbuf, L, lo, tid, nthreads);
-            lo += 2;
-        } else {
-            fwht_pass_padded<1>(fbuf, L, lo, tid, nthreads);
-            lo += 1;
-        }
-        __syncthreads();
-    }
+    fwht_row_to_lds(xp, fbuf, L, log2L, tid, nthreads);
     for (int c = tid; c < chunks; c += nthreads) {
         const float* src = fbuf + fwht_pad(8 * c);
         const f4 a = *reinterpret_cast<const f4*>(src), b = *reinterpret_cast<const f4*>(src + 4);

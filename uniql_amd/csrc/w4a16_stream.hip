@@ -36,6 +36,7 @@
 // total (old + own), stores the output and writes the word back to zero.  Integer adds
 // commute, so the result does not depend on arrival order, and nobody waits for anyone.
 #include "common.hpp"
+#include "fwht_device.hpp"
 
 namespace uniql {
 
@@ -57,6 +58,8 @@ struct StreamArgs {
     int k_valid;          // columns of X that exist (multiple of 8); the rest of K counts as zeros
     unsigned x_bytes;     // bytes from X to the end of its last row (< 2 GiB: buffer addressing)
     float had_scale;
+    int log2K;            // full-row rotation: K = 2^log2K
+    int fwht_lds;         // full-row rotation: dword offset of the rows' fp32 images in LDS
     Epilogue epi;
 };
 
@@ -70,7 +73,12 @@ struct StreamArgs {
 // uses something beyond the plain product (input shorter than K, output cut or strided, bias,
 // gated pairs); the plain instantiation leaves all of that code out, which at a few
 // microseconds per launch is measurable (instruction fetch).
-template <int RC, bool HAD, int WAVES, bool EXT>
+// HAD: 0 no rotation; 1 every 128-block of the activations is rotated in registers while it is
+// staged (zero extra memory traffic); 2 the rows are rotated as a whole (block = K, a power of
+// two): every workgroup transforms the (few) rows once, into fp32 images in LDS, while its first
+// weights are on their way, and the staging reads its 128 values from there.  Same butterfly
+// order and the same single rounding as the transform kernel: the same values bit for bit.
+template <int RC, int HAD, int WAVES, bool EXT>
 __global__ __launch_bounds__(64 * WAVES, RC == 16 ? 2 : 3)
 void w4a16_stream_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
@@ -139,6 +147,10 @@ void w4a16_stream_kernel(const StreamArgs a) {
     auto issue_loads = [&](int g, GroupRegs& r) __attribute__((always_inline)) {
 #pragma unroll
         for (int i = 0; i < XQ; ++i) {
+            if (HAD == 2) {  // the rotated rows come from LDS
+                r.xv[i] = u32x4{0u, 0u, 0u, 0u};
+                continue;
+            }
             uint32_t off = x_off[i];
             if (EXT) off = 128 * g + 8 * slot < a.k_valid ? off : 0x80000000u;
             r.xv[i] = __builtin_bit_cast(u32x4, __builtin_amdgcn_raw_buffer_load_b128(x_rsrc, off, 256u * (uint32_t)g, 0));
@@ -151,7 +163,8 @@ void w4a16_stream_kernel(const StreamArgs a) {
     };
 
     u32x4 sc_fixed = u32x4{0u, 0u, 0u, 0u};  // one scale per column: the same eight scales for every group
-    auto process = [&](const GroupRegs& r) __attribute__((always_inline)) {
+    const int fwht_row_floats = fwht_rows_image_floats(a.K);  // HAD == 2: padded fp32 image of one row
+    auto process = [&](const GroupRegs& r, int g) __attribute__((always_inline)) {
         const u32x4 scales = a.per_column ? sc_fixed : r.sc;
         // ---- rotate (optionally) and stage the activations in LDS ------------------
 #pragma unroll
@@ -159,7 +172,25 @@ void w4a16_stream_kernel(const StreamArgs a) {
             const int mrow = i * 4;
             if (mrow < a.xrows) {  // uniform
                 u32x4 v = r.xv[i];
-                if (HAD) {
+                if (HAD == 2) {
+                    v = u32x4{0u, 0u, 0u, 0u};
+                    if (mrow + kq < a.M) {
+                        const float* src = reinterpret_cast<const float*>(lds + a.fwht_lds) +
+                                           (size_t)(mrow + kq) * fwht_row_floats + fwht_pad256(128 * g + 8 * slot);
+                        const f4 lo4 = *reinterpret_cast<const f4*>(src), hi4 = *reinterpret_cast<const f4*>(src + 4);
+#pragma unroll
+                        for (int p = 0; p < 2; ++p) {
+                            h2 hv;
+                            hv.x = scaled_to_half(lo4[2 * p], a.had_scale);
+                            hv.y = scaled_to_half(lo4[2 * p + 1], a.had_scale);
+                            v[p] = h2_to_bits(hv);
+                            hv.x = scaled_to_half(hi4[2 * p], a.had_scale);
+                            hv.y = scaled_to_half(hi4[2 * p + 1], a.had_scale);
+                            v[2 + p] = h2_to_bits(hv);
+                        }
+                    }
+                }
+                if (HAD == 1) {
                     float f[8];
 #pragma unroll
                     for (int p = 0; p < 4; ++p) {
@@ -221,6 +252,12 @@ void w4a16_stream_kernel(const StreamArgs a) {
     // sequence of loads before it, so that the wait the compiler places ahead of the first use
     // of a set leaves exactly the other set's loads outstanding (a process() reached both with
     // and without a prefetch behind it would have to wait for everything).
+    // whole-row rotation: this thread's share of the activation rows is requested first (it comes
+    // from cache: every workgroup reads the same rows), so that the transform can run while the
+    // first weights, requested right behind, are still on their way
+    constexpr int kRowChunks = HAD == 2 ? 16384 / 8 / (64 * WAVES) : 1;  // 16-byte chunks of the rows per thread
+    u32x4 xin[kRowChunks];
+    if (HAD == 2) fwht_rows_load<kRowChunks>(a.X, a.ldx, a.M, a.log2K, tid, 64 * WAVES, xin);
     // the first group's loads leave before anything else is decided (a wave without groups asks
     // for the last group and ignores it)
     issue_loads(g_begin < a.G ? g_begin : a.G - 1, set_a);
@@ -235,21 +272,23 @@ void w4a16_stream_kernel(const StreamArgs a) {
         }
         sc_fixed = u32x4{t[0], t[1], t[2], t[3]};
     }
+    if (HAD == 2)  // all waves, also those without groups: the transform has workgroup barriers
+        fwht_rows_to_lds<kRowChunks>(xin, reinterpret_cast<float*>(lds + a.fwht_lds), a.M, a.K, a.log2K, tid, 64 * WAVES);
     if (g_begin < g_end) {
         int g = g_begin;
         while (g + 2 < g_end) {
             issue_loads(g + 1, set_b);
-            process(set_a);
+            process(set_a, g);
             issue_loads(g + 2, set_a);
-            process(set_b);
+            process(set_b, g + 1);
             g += 2;
         }
         if (g + 1 < g_end) {
             issue_loads(g + 1, set_b);
-            process(set_a);
-            process(set_b);
+            process(set_a, g);
+            process(set_b, g + 1);
         } else {
-            process(set_a);
+            process(set_a, g);
         }
     }
 
@@ -392,31 +431,41 @@ size_t stream_accum_bytes(int m, int n, int k) {
     return (size_t)mrows * n * sizeof(unsigned long long);
 }
 
-template <int RC, bool HAD, int WAVES, bool EXT>
-static hipError_t launch_one(const StreamArgs& a, hipStream_t stream) {
+template <int RC, int HAD, int WAVES, bool EXT>
+static hipError_t launch_one(StreamArgs a, hipStream_t stream) {
     const size_t stage = (size_t)WAVES * a.xrows * kXsStride * 4;
     const int rr_rows = a.xrows <= 4 ? 4 : (a.xrows <= 8 ? 8 : 16);
     const int wpr = 64 / rr_rows < WAVES ? 64 / rr_rows : WAVES;
     const size_t red = (size_t)wpr * rr_rows * 128 * 4;
-    const size_t shmem = stage + red;
+    size_t shmem = stage + red;
+    if (HAD == 2) {  // one padded fp32 image per activation row behind the staging and exchange areas
+        a.fwht_lds = (int)(shmem / 4);
+        shmem += (size_t)a.M * (a.K + (a.K >> 5)) * 4;
+    }
     auto kern = &w4a16_stream_kernel<RC, HAD, WAVES, EXT>;
     if (shmem > 64 * 1024) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
-                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)shmem);
-        if (e != hipSuccess) return e;
+        static bool attribute_set[64];  // per device, once per instantiation
+        int dev = 0;
+        if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipErrorInvalidDevice;
+        if (!attribute_set[dev]) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+            if (e != hipSuccess) return e;
+            attribute_set[dev] = true;
+        }
     }
     hipLaunchKernelGGL(kern, dim3(a.N / 128, a.splits), dim3(64 * WAVES), shmem, stream, a);
     return hipGetLastError();
 }
 
-template <int RC, bool HAD>
+template <int RC, int HAD>
 static hipError_t launch_waves(const StreamArgs& a, int waves, bool ext, hipStream_t stream) {
     if (waves == 8)
         return ext ? launch_one<RC, HAD, 8, true>(a, stream) : launch_one<RC, HAD, 8, false>(a, stream);
     return ext ? launch_one<RC, HAD, 4, true>(a, stream) : launch_one<RC, HAD, 4, false>(a, stream);
 }
 
-template <bool HAD>
+template <int HAD>
 static hipError_t launch_rows(const StreamArgs& a, int waves, hipStream_t stream) {
     const Epilogue& e = a.epi;
     const bool ext = e.gated || e.bias || e.residual || e.relu2 || e.transpose || e.n_store != a.N ||
@@ -428,14 +477,23 @@ static hipError_t launch_rows(const StreamArgs& a, int waves, hipStream_t stream
     return launch_waves<16, HAD>(a, waves, ext, stream);
 }
 
-// Rows are processed in slabs of at most 16; every slab re-streams the weights.
-// tune: bits 0..7 groups per wave, bits 8..12 waves per workgroup (4 or 8); zero fields mean
-// "choose".
 // the activation rows of a 16-row slab are addressed with 32-bit byte offsets
 bool stream_shape_ok(int k, int64_t lda) { return (15 * lda + k) * 2 < ((int64_t)1 << 31); }
 
+// Whether the full-row rotation (block = k) of an m-row call runs inside the streaming kernel:
+// k a power of two and the rows' fp32 images (k + k/16 floats each, per 16-row slab) small enough
+// to leave room for several workgroups per compute unit.
+bool stream_rotates_rows(int m, int k) {
+    const int mm = m < 16 ? m : 16;
+    return k >= 256 && (k & (k - 1)) == 0 && (int64_t)mm * k <= 16384;
+}
+
+// Rows are processed in slabs of at most 16; every slab re-streams the weights.
+// had_mode: 0 no rotation, 1 128-blocks, 2 whole rows (stream_rotates_rows must hold, k_valid = k).
+// tune: bits 0..7 groups per wave, bits 8..12 waves per workgroup (4 or 8); zero fields mean
+// "choose".
 int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const void* S, void* D,
-                  const Epilogue& epi, void* accum, int m, int n, int k, int groups, bool had128, float had_scale,
+                  const Epilogue& epi, void* accum, int m, int n, int k, int groups, int had_mode, float had_scale,
                   unsigned tune, hipStream_t stream) {
     if (!stream_shape_ok(k, lda)) return UNIQL_E_SHAPE;
     StreamArgs a;
@@ -450,6 +508,9 @@ int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const 
     a.k_valid = k_valid;
     a.epi = epi;
     a.had_scale = had_scale;
+    a.fwht_lds = 0;
+    a.log2K = 0;
+    while ((1 << a.log2K) < k) ++a.log2K;
     int waves_override = (int)((tune >> 8) & 0x1fu);
     if (waves_override != 4 && waves_override != 8) waves_override = 0;
     const size_t out_elt = epi.out_f32 ? 4 : 2;
@@ -464,7 +525,9 @@ int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const 
         a.X = reinterpret_cast<const half_t*>(A) + (size_t)m0 * lda;
         a.D = reinterpret_cast<char*>(D) + (size_t)m0 * (epi.transpose ? 1 : epi.ldd) * out_elt;
         if (epi.residual) a.epi.residual = epi.residual + (size_t)m0 * epi.ldr;
-        const hipError_t e = had128 ? launch_rows<true>(a, plan.waves, stream) : launch_rows<false>(a, plan.waves, stream);
+        const hipError_t e = had_mode == 1   ? launch_rows<1>(a, plan.waves, stream)
+                             : had_mode == 2 ? launch_rows<2>(a, plan.waves, stream)
+                                             : launch_rows<0>(a, plan.waves, stream);
         if (e != hipSuccess) return UNIQL_E_LAUNCH;
     }
     return UNIQL_OK;
