@@ -321,6 +321,21 @@ enum { UNIQL_DT_F16 = 0, UNIQL_DT_BF16 = 1, UNIQL_DT_F32 = 2 };
 int uniql_fwht(const void* x, void* y, int64_t rows, int dim, int block,
                float scale, int dtype, void* stream);
 
+/*
+ * y[r, :] = round((x[r, :] . (H_base (x) H_P)) * scale) for dim = base * P, base in {12, 20, 28, 40}, P a power
+ * of two: the row is `base` chunks of P values, every chunk gets the P-point transform, then the
+ * base x base Hadamard matrix combines the chunks (y[c P + i] = sum_c' z[c' P + i] H[c'][c]); fp32
+ * throughout, one rounding at the end.  Replaces fast_hadamard_transform_cuda.fast_hadamard_transform_{12,20,28,40}N
+ * as selected by quantize/hadamard_helpers.py:20-31 (Qwen2's 3584 = 28 * 128, Llama's 14336 = 28 * 512).
+ * The base matrices of that third-party package are not part of the reference tree; the ones used here
+ * (Sloane's 12 x 12, Paley's constructions for 20 and 28, the doubled 20 for 40) satisfy H H^T = base I,
+ * which is all that HadLinear and the Hadamard module need as long as both sides of a layer use this
+ * library; results are NOT guaranteed to match weights rotated offline with the reference's tables.
+ *   x, y   device, [rows, dim] contiguous, element type `dtype`; y may equal x;  dim <= 40960
+ */
+int uniql_fwht_composite(const void* x, void* y, int64_t rows, int dim, int base,
+                         float scale, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -33,9 +33,14 @@ Pinning status (what proves each function right, besides reading):
     rotation in float64 for identity indices, an independently permuted frequency table,
     norm preservation, and torch's fp16 CPU arithmetic for the order of the roundings
   * power-of-two Hadamard .................... scipy.linalg.hadamard, involution,
-    Parseval.  The 12N/20N/28N/40N variants need base matrices that live in an
-    un-vendored third-party package (Dao-AILab fast-hadamard-transform, commit
-    unknown): they are not restated here and are "parity unpinned".
+    Parseval.
+  * composite Hadamard widths (12N/20N/28N/40N, `fwht_composite`) ... PARITY UNPINNED against
+    the reference: its base matrices live in an un-vendored third-party package
+    (Dao-AILab fast-hadamard-transform, commit unknown; submodule empty in the
+    reference tree).  What is pinned is the mathematics: the matrices built here
+    (Sloane's 12 x 12, Paley I over GF(19), Paley II over GF(13), the doubled 20) satisfy
+    H H^T = n I, the transform equals x @ kron(H_base, H_P) in float64, and
+    HadLinear's fused and lazy forms agree.
 """
 from __future__ import annotations
 
@@ -403,10 +408,74 @@ def fwht(x: np.ndarray, scale: float, block: int | None = None,
     return y.reshape(x.shape).astype(x.dtype)
 
 
+def _legendre(a: int, q: int) -> int:
+    a %= q
+    if a == 0:
+        return 0
+    return 1 if pow(a, (q - 1) // 2, q) == 1 else -1
+
+
+def hadamard_base_matrix(base: int) -> np.ndarray:
+    """The base x base Hadamard matrix behind fast_hadamard_transform_{base}N
+    (hadamard_helpers.py:20-31).  The reference's own tables are not in its tree (parity
+    unpinned); these are textbook constructions: 12 Sloane's "had.12" (first row + - ... -, the
+    other rows cyclic shifts of + + - + - - - + + + - + behind a leading +), 20 Paley I over
+    GF(19), 28 Paley II over GF(13), 40 the Sylvester doubling of the 20."""
+    if base == 12:
+        core = [1, -1, 1, -1, -1, -1, 1, 1, 1, -1, 1]
+        h = np.ones((12, 12), dtype=np.int64)
+        h[0, 1:] = -1
+        for r in range(11):
+            h[1 + r, 1:] = np.roll(core, r)
+        return h
+    if base == 20:
+        q = 19
+        jac = np.array([[_legendre(i - j, q) for j in range(q)] for i in range(q)], dtype=np.int64)
+        s = np.zeros((q + 1, q + 1), dtype=np.int64)
+        s[0, 1:] = 1
+        s[1:, 0] = -1
+        s[1:, 1:] = jac
+        return s + np.eye(q + 1, dtype=np.int64)
+    if base == 28:
+        q = 13
+        jac = np.array([[_legendre(i - j, q) for j in range(q)] for i in range(q)], dtype=np.int64)
+        s = np.zeros((q + 1, q + 1), dtype=np.int64)
+        s[0, 1:] = 1
+        s[1:, 0] = 1
+        s[1:, 1:] = jac
+        eye = np.eye(q + 1, dtype=np.int64)
+        return np.block([[s + eye, s - eye], [s - eye, -s - eye]])
+    if base == 40:
+        h20 = hadamard_base_matrix(20)
+        return np.block([[h20, h20], [h20, -h20]])
+    raise ValueError(f"no base matrix of order {base}")
+
+
+def fwht_composite(x: np.ndarray, scale: float, base: int, acc=np.float32) -> np.ndarray:
+    """y = (x . (H_base (x) H_P)) * scale along the last axis of width base * P: the P-point
+    transform inside each of the `base` chunks, then the base matrix across the chunks, added in
+    ascending chunk order; arithmetic in `acc`, one rounding to x's dtype.  The contract of
+    fast_hadamard_transform_{12,20,28,40}N(x, scale) as called at hadamard_helpers.py:20-31,45."""
+    dim = x.shape[-1]
+    p = dim // base
+    assert base * p == dim and is_pow2(p)
+    z = fwht(np.asarray(x).astype(acc), 1.0, block=p, acc=acc).reshape(-1, base, p)
+    h = hadamard_base_matrix(base)
+    y = np.zeros_like(z)
+    for c in range(base):
+        total = np.zeros((z.shape[0], p), dtype=acc)
+        for cp in range(base):
+            total = total + (z[:, cp, :] if h[cp, c] > 0 else -z[:, cp, :])
+        y[:, c, :] = total
+    y = y * acc(scale)
+    return y.reshape(x.shape).astype(x.dtype)
+
+
 def hadamard_module_forward(x: np.ndarray, dim: int) -> np.ndarray:
     """Hadamard(dim).forward(x).  quant_hadamard_layers.py:5-21."""
     base, scale = had_variant(dim)
-    assert base == 2, "non power-of-two variants are not restated (parity unpinned)"
+    if base != 2:
+        return fwht_composite(x, scale, base)
     return fwht(x, scale)
 
 

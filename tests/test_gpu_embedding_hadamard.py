@@ -111,5 +111,49 @@ def test_hadamard_module_and_involution(gpu):
     assert float((back.float() - x.float()).abs().max()) < 5e-3
     with pytest.raises(AssertionError):
         Hadamard(12160)
-    with pytest.raises(NotImplementedError):
-        Hadamard(14336)(torch.zeros(1, 14336, dtype=torch.float16, device=gpu))
+    assert Hadamard(14336).N == 28 and Hadamard(3584).N == 28 and Hadamard(5120).N == 40
+
+
+@pytest.mark.parametrize("dim", [12, 24, 1536, 20, 1280, 28, 3584, 14336, 40, 10240, 40960])
+@pytest.mark.parametrize("dtype", ["float16", "bfloat16", "float32"])
+def test_composite_hadamard_widths(gpu, dim, dtype):
+    """fast_hadamard_transform_{12,20,28,40}N: bit for bit the oracle's fp32 arithmetic (same chunk
+    transforms, same ascending sum over the base matrix, one rounding), and the module / helper
+    pick the variant by width as the reference does.  The reference's own base matrices are not in
+    its tree: parity with it is unpinned, the oracle pins the mathematics (tests/test_oracle_golden.py)."""
+    from uniql_amd.quantize.hadamard_helpers import get_had_fn, had_transform
+    fn, base, scale = get_had_fn(dim)
+    assert base == O.had_variant(dim)[0] and base in (12, 20, 28, 40) and fn.__name__ == f"fast_hadamard_transform_{base}N"
+    tdt = getattr(torch, dtype)
+    x = torch.randn(3, dim, generator=torch.Generator().manual_seed(dim)).to(tdt)
+    y = fn(x.to(gpu), scale)
+    assert y.dtype == tdt and y.shape == x.shape
+    if dtype == "bfloat16":     # numpy has no bfloat16: round the oracle's fp32 result with torch
+        want32 = O.fwht_composite(x.float().numpy(), 1.0, base)
+        want = (torch.from_numpy(want32) * torch.tensor(scale, dtype=torch.float32)).to(torch.bfloat16)
+        assert torch.equal(y.cpu(), want)
+    else:
+        want = O.fwht_composite(x.numpy(), scale, base)
+        assert np.array_equal(y.cpu().numpy().view(np.uint8), want.view(np.uint8))
+    assert torch.equal(had_transform(x.to(gpu).view(3, 1, dim)).view(3, dim), y)
+
+
+@pytest.mark.parametrize("din,dout", [(3584, 512), (1536, 14336), (1280, 640)])
+def test_hadlinear_with_composite_widths(gpu, din, dout):
+    """HadLinear on widths 28 * 128, 12 * 128, 28 * 512, 20 * 64, 20 * 32: rotating the input undoes the input-side
+    rotation of the weight (H H^T = n I), the fused and the lazy form agree."""
+    from uniql_amd.quantize.hadamard_helpers import get_had_fn
+    from uniql_amd.quantize.quant_linear_layers import HadLinear
+    g = torch.Generator().manual_seed(din + dout)
+    lin = torch.nn.Linear(din, dout, bias=False).half().to(gpu)
+    lin.weight.data = (torch.randn(dout, din, generator=g) * 0.05).half().to(gpu)
+    x = torch.randn(4, din, generator=g).half().to(gpu)
+    lazy = HadLinear(lin, input_transform=True, output_transform=True)
+    fused = HadLinear(lin, input_transform=True, output_transform=True, fuse_had=True)
+    fn_in, _, s_in = get_had_fn(din)
+    fn_out, _, s_out = get_had_fn(dout)
+    y_lazy, y_fused = lazy(fn_in(x, s_in)), fused(fn_in(x, s_in))
+    assert float((y_lazy.float() - y_fused.float()).abs().max()) < 2e-2
+    # y = (x H_in / sqrt(n)) (H_out^T W H_in / sqrt(n m))^T = (x W^T) H_out / sqrt(m): the plain product, output rotated
+    want = fn_out(lin(x).float(), s_out)
+    assert float((y_fused.float() - want).abs().max()) < 3e-2

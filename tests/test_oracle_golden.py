@@ -295,3 +295,36 @@ def test_hadlinear_identity():
     assert np.allclose(wh, w @ h, atol=1e-5)
     who = O.hadlinear_fused_weight(np.ascontiguousarray(w.T), False, True)   # [64, 24] output side
     assert np.allclose(who, h @ w.T, atol=1e-5)
+
+
+@pytest.mark.parametrize("base", [12, 20, 28, 40])
+def test_hadamard_base_matrices_are_hadamard(base):
+    """Entries +-1, H H^T = H^T H = n I; the 12 is Sloane's had.12 written out."""
+    h = O.hadamard_base_matrix(base)
+    assert h.shape == (base, base) and set(np.unique(h)) == {-1, 1}
+    assert np.array_equal(h @ h.T, base * np.eye(base, dtype=np.int64))
+    assert np.array_equal(h.T @ h, base * np.eye(base, dtype=np.int64))
+    if base == 12:
+        rows = ["+-----------", "++-+---+++-+", "+++-+---+++-", "+-++-+---+++", "++-++-+---++", "+++-++-+---+",
+                "++++-++-+---", "+-+++-++-+--", "+--+++-++-+-", "+---+++-++-+", "++---+++-++-", "+-+---+++-++"]
+        assert np.array_equal(h, np.array([[1 if c == "+" else -1 for c in r] for r in rows]))
+    if base == 40:
+        h20 = O.hadamard_base_matrix(20)
+        assert np.array_equal(h[:20, 20:], h20) and np.array_equal(h[20:, 20:], -h20)
+
+
+@pytest.mark.parametrize("dim", [12, 96, 160, 448, 1280])
+def test_composite_transform_is_the_kronecker_product(dim):
+    """fwht_composite(x) = x @ kron(H_base, H_P) (float64 matmul with scipy's Sylvester matrix), its rows are
+    orthogonal (x -> transform -> transform with the transposed matrix gives dim * x)."""
+    from scipy.linalg import hadamard
+    base = O.had_variant(dim)[0]
+    p = dim // base
+    big = np.kron(O.hadamard_base_matrix(base), hadamard(p) if p > 1 else np.ones((1, 1)))
+    x = np.random.default_rng(dim).standard_normal((5, dim))
+    got = O.fwht_composite(x, 1.0, base, acc=np.float64)
+    assert np.allclose(got, x @ big, rtol=0, atol=1e-9)
+    assert np.allclose(got @ big.T, dim * x, rtol=0, atol=1e-8)
+    x16 = x.astype(np.float16)
+    y16 = O.fwht_composite(x16, dim ** -0.5, base)
+    assert y16.dtype == np.float16 and np.abs(y16.astype(np.float64) - (x16.astype(np.float64) @ big) * dim ** -0.5).max() < 4e-3

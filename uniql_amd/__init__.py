@@ -30,7 +30,7 @@ def install_extension_aliases() -> None:
     had = types.ModuleType("fast_hadamard_transform_cuda")
     had.fast_hadamard_transform = ops.fast_hadamard_transform
     for n in (12, 20, 28, 40):
-        setattr(had, f"fast_hadamard_transform_{n}N", ops.unsupported_hadamard_variant(n))
+        setattr(had, f"fast_hadamard_transform_{n}N", ops.composite_hadamard_variant(n))
     sys.modules.setdefault("quant_linear_cuda", lin)
     sys.modules.setdefault("quant_embedding_cuda", emb)
     sys.modules.setdefault("fast_hadamard_transform_cuda", had)

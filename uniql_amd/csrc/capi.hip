@@ -31,6 +31,8 @@ int rope_indices_launch(void* q, int64_t q_row_stride, void* k, int64_t k_row_st
                         int cos_batch, int n_qh, int n_kh, int hd, int cos_dim, hipStream_t stream);
 int fwht_launch(const void* x, void* y, int64_t rows, int dim, int block, float scale, int dtype,
                 hipStream_t stream);
+int fwht_composite_launch(const void* x, void* y, int64_t rows, int dim, int base, float scale, int dtype,
+                          hipStream_t stream);
 int quantize_launch(const void* W, int64_t ldw, const void* given_scales, void* B, void* S, int out_features,
                     int in_features, int n_pad, int k_pad, hipStream_t stream);
 int pack_launch(const uint8_t* codes, const void* scales, void* B, void* S, int n, int k, int n_pad, int k_pad,
@@ -416,6 +418,15 @@ int uniql_fwht(const void* x, void* y, int64_t rows, int dim, int block, float s
     if (!x || !y) return UNIQL_E_NULL;
     if (block == 128 && dtype == UNIQL_DT_F16 && (!aligned16(x) || !aligned16(y))) return UNIQL_E_ALIGN;
     return fwht_launch(x, y, rows, dim, block, scale, dtype, reinterpret_cast<hipStream_t>(stream));
+}
+
+int uniql_fwht_composite(const void* x, void* y, int64_t rows, int dim, int base, float scale, int dtype, void* stream) {
+    if (dtype != UNIQL_DT_F16 && dtype != UNIQL_DT_BF16 && dtype != UNIQL_DT_F32) return UNIQL_E_UNSUPPORTED;
+    if (base != 12 && base != 20 && base != 28 && base != 40) return UNIQL_E_UNSUPPORTED;
+    if (rows < 0 || dim <= 0 || dim % base != 0 || !is_pow2(dim / base) || dim > 40960) return UNIQL_E_SHAPE;
+    if (rows == 0) return UNIQL_OK;
+    if (!x || !y) return UNIQL_E_NULL;
+    return fwht_composite_launch(x, y, rows, dim, base, scale, dtype, reinterpret_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -3,6 +3,7 @@
 // Butterflies run in fp32, lowest index bit first, one rounding to fp16 at the end.
 #include "common.hpp"
 #include "fwht_device.hpp"
+#include "hadamard_base.hpp"
 
 namespace uniql {
 
@@ -240,6 +241,90 @@ static int fwht_f16_launch(const void* x, void* y, int64_t pieces, int block, fl
     hipLaunchKernelGGL(fwht_f16_kernel, dim3((unsigned)pieces), dim3(threads), shmem, stream,
                        reinterpret_cast<const u32x4*>(x), reinterpret_cast<u32x4*>(y), block, log2L, scale);
     return UNIQL_OK;
+}
+
+// ---- composite widths: dim = BASE * P with P a power of two -----------------------------------
+// The row is BASE chunks of P values: every chunk gets the P-point transform (LDS passes over
+// the whole row touch only index bits below log2 P, so the chunks stay apart), then the BASE x BASE
+// matrix combines the chunks: y[c P + i] = sum_c' z[c' P + i] H[c'][c], added in ascending c' in
+// fp32; one rounding at the end.
+template <typename T, int BASE>
+__global__ __launch_bounds__(256) void fwht_composite_kernel(const T* __restrict__ x, T* __restrict__ y, int P,
+                                                            int log2P, float scale) {
+    extern __shared__ __attribute__((aligned(16))) float fbuf[];
+    const uint64_t* table = BASE == 12 ? kHadamard12 : BASE == 20 ? kHadamard20 : BASE == 28 ? kHadamard28 : kHadamard40;
+    const int tid = threadIdx.x;
+    const int L = BASE * P;
+    const T* xp = x + (size_t)blockIdx.x * L;
+    T* yp = y + (size_t)blockIdx.x * L;
+    for (int i = tid; i < L; i += 256) fbuf[i] = (float)xp[i];
+    __syncthreads();
+    int lo = 0;
+    while (lo < log2P) {
+        const int left = log2P - lo;
+        if (left >= 3) {
+            fwht_pass<3>(fbuf, L, lo, tid, 256);
+            lo += 3;
+        } else if (left == 2) {
+            fwht_pass<2>(fbuf, L, lo, tid, 256);
+            lo += 2;
+        } else {
+            fwht_pass<1>(fbuf, L, lo, tid, 256);
+            lo += 1;
+        }
+        __syncthreads();
+    }
+    for (int i = tid; i < P; i += 256) {
+        float z[BASE];
+#pragma unroll
+        for (int c = 0; c < BASE; ++c) z[c] = fbuf[c * P + i];
+#pragma unroll
+        for (int c = 0; c < BASE; ++c) {
+            const uint64_t minus = table[c];
+            float sum = 0.f;
+#pragma unroll
+            for (int cp = 0; cp < BASE; ++cp) sum += ((minus >> cp) & 1ull) ? -z[cp] : z[cp];
+            float p = sum * scale;
+            asm volatile("" : "+v"(p));  // see scaled_to_half: keep multiply and rounding separate
+            yp[c * P + i] = (T)p;
+        }
+    }
+}
+
+template <typename T, int BASE>
+static int fwht_composite_go(const void* x, void* y, int64_t rows, int P, float scale, hipStream_t stream) {
+    int log2P = 0;
+    while ((1 << log2P) < P) ++log2P;
+    const size_t shmem = (size_t)BASE * P * sizeof(float);
+    auto kern = &fwht_composite_kernel<T, BASE>;
+    if (shmem > 64 * 1024 &&
+        hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            (int)shmem) != hipSuccess)
+        return UNIQL_E_LAUNCH;
+    hipLaunchKernelGGL(kern, dim3((unsigned)rows), dim3(256), shmem, stream, reinterpret_cast<const T*>(x),
+                       reinterpret_cast<T*>(y), P, log2P, scale);
+    return hipGetLastError() == hipSuccess ? UNIQL_OK : UNIQL_E_LAUNCH;
+}
+
+template <typename T>
+static int fwht_composite_base(const void* x, void* y, int64_t rows, int base, int P, float scale, hipStream_t stream) {
+    switch (base) {
+        case 12: return fwht_composite_go<T, 12>(x, y, rows, P, scale, stream);
+        case 20: return fwht_composite_go<T, 20>(x, y, rows, P, scale, stream);
+        case 28: return fwht_composite_go<T, 28>(x, y, rows, P, scale, stream);
+        case 40: return fwht_composite_go<T, 40>(x, y, rows, P, scale, stream);
+        default: return UNIQL_E_UNSUPPORTED;
+    }
+}
+
+int fwht_composite_launch(const void* x, void* y, int64_t rows, int dim, int base, float scale, int dtype,
+                          hipStream_t stream) {
+    if (rows == 0) return UNIQL_OK;
+    if (rows > 0x7fffffffLL) return UNIQL_E_SHAPE;
+    const int P = dim / base;
+    if (dtype == UNIQL_DT_F16) return fwht_composite_base<half_t>(x, y, rows, base, P, scale, stream);
+    if (dtype == UNIQL_DT_BF16) return fwht_composite_base<__bf16>(x, y, rows, base, P, scale, stream);
+    return fwht_composite_base<float>(x, y, rows, base, P, scale, stream);
 }
 
 template <typename T>

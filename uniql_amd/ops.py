@@ -20,7 +20,7 @@ from . import _capi
 
 __all__ = [
     "w4a16o16_gemm", "w4a16_gemm_ex", "w4a16_gemm_static", "w4a16_linear", "w4a16_dequant", "w4a16_embedding_lookup",
-    "fast_hadamard_transform", "hadamard_blockwise", "unsupported_hadamard_variant",
+    "fast_hadamard_transform", "hadamard_blockwise", "hadamard_composite", "composite_hadamard_variant",
     "w4a16_read_floor", "w4a16_quantize", "w4a16_pack", "w4a16_unpack", "w4_embedding_quantize", "rope_indices_",
 ]
 
@@ -511,10 +511,30 @@ def fast_hadamard_transform(x: torch.Tensor, scale: float = 1.0) -> torch.Tensor
     return hadamard_blockwise(x, scale, dim)
 
 
-def unsupported_hadamard_variant(base: int):
+def hadamard_composite(x: torch.Tensor, scale: float, base: int) -> torch.Tensor:
+    """(x . (H_base (x) H_P)) * scale along the last axis of width base * P, P a power of two
+    (uniql_fwht_composite); new tensor."""
+    _require_gpu(x, "x")
+    dim = x.shape[-1]
+    dtypes = {torch.float16: _capi.DT_F16, torch.bfloat16: _capi.DT_BF16, torch.float32: _capi.DT_F32}
+    if x.dtype not in dtypes:
+        raise RuntimeError(f"hadamard transform supports float16 / bfloat16 / float32, got {x.dtype}")
+    lib = _capi.load()
+    xc = x.contiguous()
+    dev = x.device
+    with _device_guard(dev):
+        y = torch.empty_like(xc)
+        rows = xc.numel() // dim if dim else 0
+        code = lib.uniql_fwht_composite(xc.data_ptr(), y.data_ptr(), rows, dim, base, float(scale),
+                                        dtypes[x.dtype], _stream_ptr(dev))
+    _capi.check(code, "uniql_fwht_composite")
+    return y
+
+
+def composite_hadamard_variant(base: int):
+    """The transform fast_hadamard_transform_{base}N(x, scale) of the reference's extension, for widths
+    base * 2^k (quantize/hadamard_helpers.py:20-31)."""
     def _fn(x, scale=1.0):
-        raise NotImplementedError(
-            f"fast_hadamard_transform_{base}N: the {base}x{base} base matrix comes from a third-party "
-            "package that is not part of the reference tree; only power-of-two widths are implemented")
+        return hadamard_composite(x, scale, base)
     _fn.__name__ = f"fast_hadamard_transform_{base}N"
     return _fn

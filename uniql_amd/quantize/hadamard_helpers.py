@@ -20,12 +20,12 @@ def prev_power_of_two(x: int) -> int:
 
 def get_had_fn(dim: int):
     """(transform, base N, scale): widths 40*2^k, 28*2^k, 20*2^k, 12*2^k pick the
-    composite variants (not implemented here: they raise when called), every
-    other width must be a power of two (hadamard_helpers.py:18-36)."""
+    composite variants, every other width must be a power of two
+    (hadamard_helpers.py:18-36)."""
     scale = 1.0 / math.sqrt(dim)
     for base in (40, 28, 20, 12):
         if dim % base == 0 and is_pow2(dim // base):
-            return ops.unsupported_hadamard_variant(base), base, scale
+            return ops.composite_hadamard_variant(base), base, scale
     assert is_pow2(dim), f"Invalid dim: {dim}. dim must be a power of 2."
     return ops.fast_hadamard_transform, 2, scale
 
