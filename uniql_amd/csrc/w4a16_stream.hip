@@ -548,9 +548,8 @@ void w4a16_read_floor_kernel(const u32x4* B, const half_t* S, int N, int G, int 
     const int lane = tid & 63;
     const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int slot = lane & 15, kq = lane >> 4, c8 = slot & 7;
-    const int nstrips = N >> 7;
-    const int strip = blockIdx.x % nstrips;
-    const int split = blockIdx.x / nstrips;
+    const int strip = blockIdx.x;
+    const int split = blockIdx.y;
     const int N4 = N >> 1;
     const int g_begin = (split * WAVES + w) * upw;
     const int g_end = (g_begin + upw < G) ? (g_begin + upw) : G;
@@ -576,18 +575,18 @@ void w4a16_read_floor_kernel(const u32x4* B, const half_t* S, int N, int G, int 
             for (int rr = 0; rr < 8; ++rr) x ^= wq[d][rr];
         }
     }
-    if ((x[0] ^ x[1] ^ x[2] ^ x[3]) == 0x9e3779b9u) sink[blockIdx.x * WAVES + w] = x[0];
+    if ((x[0] ^ x[1] ^ x[2] ^ x[3]) == 0x9e3779b9u) sink[(blockIdx.y * gridDim.x + blockIdx.x) * WAVES + w] = x[0];
 }
 
 template <int WAVES>
-static void read_floor_depth(int depth, int grid, hipStream_t stream, const u32x4* B, const half_t* S, int N, int G,
+static void read_floor_depth(int depth, dim3 grid, hipStream_t stream, const u32x4* B, const half_t* S, int N, int G,
                              int upw, uint32_t* sink) {
     if (depth >= 4)
-        hipLaunchKernelGGL((w4a16_read_floor_kernel<WAVES, 4>), dim3(grid), dim3(64 * WAVES), 0, stream, B, S, N, G, upw, sink);
+        hipLaunchKernelGGL((w4a16_read_floor_kernel<WAVES, 4>), grid, dim3(64 * WAVES), 0, stream, B, S, N, G, upw, sink);
     else if (depth >= 2)
-        hipLaunchKernelGGL((w4a16_read_floor_kernel<WAVES, 2>), dim3(grid), dim3(64 * WAVES), 0, stream, B, S, N, G, upw, sink);
+        hipLaunchKernelGGL((w4a16_read_floor_kernel<WAVES, 2>), grid, dim3(64 * WAVES), 0, stream, B, S, N, G, upw, sink);
     else
-        hipLaunchKernelGGL((w4a16_read_floor_kernel<WAVES, 1>), dim3(grid), dim3(64 * WAVES), 0, stream, B, S, N, G, upw, sink);
+        hipLaunchKernelGGL((w4a16_read_floor_kernel<WAVES, 1>), grid, dim3(64 * WAVES), 0, stream, B, S, N, G, upw, sink);
 }
 
 // tune: as stream_launch (bits 0..7 groups per wave, bits 8..12 waves per workgroup), plus bits
@@ -597,7 +596,7 @@ int read_floor_launch(const void* B, const void* S, void* sink, int m, int n, in
     if (waves_override != 4 && waves_override != 8) waves_override = 0;
     const StreamPlan plan = stream_plan(m < 16 ? m : 16, n, k, (int)(tune & 0xffu), waves_override);
     const int depth = (int)((tune >> 13) & 7u);
-    const int grid = (n / 128) * plan.splits;
+    const dim3 grid(n / 128, plan.splits);
     if (plan.waves == 8)
         read_floor_depth<8>(depth, grid, stream, reinterpret_cast<const u32x4*>(B), reinterpret_cast<const half_t*>(S), n,
                             k / 128, plan.upw, reinterpret_cast<uint32_t*>(sink));
