@@ -167,27 +167,23 @@ __global__ __launch_bounds__(512) void fwht_f16_wide_kernel(const u32x4* __restr
         *reinterpret_cast<f4*>(dst + 4) = f4{f[4], f[5], f[6], f[7]};
     }
     __syncthreads();
-    int lo = 3;
-    const int top = log2L - 5;  // first bit of the final phase
-    while (lo < top) {
-        const int left = top - lo;
-        if (left >= 5) {
-            fwht_pass_padded<5>(fbuf, L, lo, tid, nthreads);
-            lo += 5;
-        } else if (left == 4) {
-            fwht_pass_padded<4>(fbuf, L, lo, tid, nthreads);
-            lo += 4;
-        } else if (left == 3) {
-            fwht_pass_padded<3>(fbuf, L, lo, tid, nthreads);
-            lo += 3;
-        } else if (left == 2) {
-            fwht_pass_padded<2>(fbuf, L, lo, tid, nthreads);
-            lo += 2;
-        } else {
-            fwht_pass_padded<1>(fbuf, L, lo, tid, nthreads);
-            lo += 1;
-        }
-        __syncthreads();
+    // index bits 3 .. log2L - 6 (log2L = 12 .. 15), then the top five bits in the final phase
+    switch (log2L) {
+        case 12: fwht_pass_fixed<4, 3>(fbuf, L, tid, nthreads); __syncthreads(); break;
+        case 13: fwht_pass_fixed<5, 3>(fbuf, L, tid, nthreads); __syncthreads(); break;
+        case 14:
+            fwht_pass_fixed<5, 3>(fbuf, L, tid, nthreads);
+            __syncthreads();
+            fwht_pass_fixed<1, 8>(fbuf, L, tid, nthreads);
+            __syncthreads();
+            break;
+        case 15:
+            fwht_pass_fixed<5, 3>(fbuf, L, tid, nthreads);
+            __syncthreads();
+            fwht_pass_fixed<2, 8>(fbuf, L, tid, nthreads);
+            __syncthreads();
+            break;
+        default: break;
     }
     // final phase: values 2 tid, 2 tid + 1 at the 32 strides of L / 32
     const int stride = L >> 5;

@@ -41,21 +41,19 @@ __device__ __forceinline__ void fwht_pass_padded(float* buf, int L, int lo, int 
 }
 
 // The same with the first bit known at compile time: every address of a task is the first one
-// plus a constant (the padding term is linear inside a task: for LO >= 7 a step of 2^LO adds whole
-// 128-blocks, for LO == 3 with CNT <= 4 a task stays inside one 128-block), so the index arithmetic
-// is done once per task instead of once per value.
+// plus a constant (the task's values lie (i << LO) apart and those bits of the first index are zero,
+// so the padding term of value i is that of the first index plus ((i << LO) >> 7) << 3): the index
+// arithmetic is done once per task instead of once per value.
 template <int CNT, int LO>
 __device__ __forceinline__ void fwht_pass_fixed(float* buf, int L, int tid, int nthreads) {
-    static_assert(LO >= 7 || (LO == 3 && CNT <= 4), "padding term must be linear inside a task");
     constexpr int E = 1 << CNT;
-    constexpr int STEP = LO >= 7 ? (1 << LO) + (1 << (LO - 4)) : (1 << LO);  // padded distance of two values
     const int tasks = L >> CNT;
     constexpr int lowmask = (1 << LO) - 1;
     for (int t = tid; t < tasks; t += nthreads) {
         float* p0 = buf + fwht_pad(((t >> LO) << (LO + CNT)) | (t & lowmask));
         float v[E];
 #pragma unroll
-        for (int i = 0; i < E; ++i) v[i] = p0[i * STEP];
+        for (int i = 0; i < E; ++i) v[i] = p0[(i << LO) + (((i << LO) >> 7) << 3)];
 #pragma unroll
         for (int h = 1; h < E; h <<= 1) {
 #pragma unroll
@@ -68,7 +66,7 @@ __device__ __forceinline__ void fwht_pass_fixed(float* buf, int L, int tid, int 
             }
         }
 #pragma unroll
-        for (int i = 0; i < E; ++i) p0[i * STEP] = v[i];
+        for (int i = 0; i < E; ++i) p0[(i << LO) + (((i << LO) >> 7) << 3)] = v[i];
     }
 }
 

@@ -332,9 +332,12 @@ void w4a16_stream_kernel(const StreamArgs a) {
         for (int i = 0; i < NI; ++i) {
             const int ml = (tid >> 7) + RPT * i;
             if (ml < a.M) {
-                for (int ww = 0; ww < wpr; ++ww) {
-                    tot[i] += red[(ww * rr_rows + ml) * 128 + col_out];
-                    if (gated) oth[i] += red[(ww * rr_rows + ml) * 128 + col_pair];
+#pragma unroll
+                for (int ww = 0; ww < WAVES; ++ww) {
+                    if (ww < wpr) {
+                        tot[i] += red[(ww * rr_rows + ml) * 128 + col_out];
+                        if (gated) oth[i] += red[(ww * rr_rows + ml) * 128 + col_pair];
+                    }
                 }
             }
         }
