@@ -106,8 +106,7 @@ int uniql_stream_capture_id(void* stream, unsigned long long* id);
  * gives an infinite fp16 result; with UNIQL_F_OUT_F32 the clamp itself is visible).  A NaN
  * partial sum makes the result NaN, as without a K split.  The one difference from a launch
  * that does not split K: +inf and -inf that meet from DIFFERENT workgroups cancel to a finite
- * value instead of NaN.  (An infinite ACTIVATION gives NaN in the streaming kernel with or
- * without a split: the zero point enters as a separate -8 * sum(x) term.)  Either kernel's result is the same from run to run: integer additions
+ * value instead of NaN.  Either kernel's result is the same from run to run: integer additions
  * in the first, partial tiles added in split order in the second.
  */
 size_t uniql_w4a16_gemm_accum_bytes(int m, int n, int k);
