@@ -106,6 +106,9 @@ def test_argument_checks_need_no_gpu(lib):
     fake = ctypes.c_void_p(0x10000)
     assert call(A=fake, B=fake, S=fake, D=fake, m=17, n=128, k=128, k_in=128, groups=1, ldd=128, n_out=128,
                 lda=1 << 24) == -2
+    # the streaming kernel addresses a 16-row slab of activations with 32-bit byte offsets
+    assert call(A=fake, B=fake, S=fake, D=fake, m=2, n=128, k=128, k_in=128, groups=1, ldd=128, n_out=128,
+                lda=1 << 27) == -2
     assert lib.uniql_w4a16_linear_temp_bytes(3, 4096, 4096, 4000, 0) == 3 * 4096 * 2
     assert lib.uniql_w4a16_linear_temp_bytes(3, 4096, 4096, 4096, 0) == 0
     r = lib.uniql_rope_indices
