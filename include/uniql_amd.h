@@ -48,8 +48,10 @@ enum {
                                       untouched; uniql_w4a16_linear takes ldd >= m from the caller */
     /* tuning hooks, 0 = choose.  Streaming kernel: bits 8..15 K-groups per wavefront,
        bits 16..20 wavefronts per workgroup (4 or 8).
-       Tiled kernel: bits 8..15 number of K splits over workgroups, bits 16..19 row tiles of 32
-       per workgroup (1, 2 or 4), bits 20..21 wave quartets per workgroup (1 or 2). */
+       Tiled kernels: bits 8..15 number of K splits over workgroups, bits 16..19 row tiles of 32
+       per workgroup (1, 2 or 4: the 128-column kernel; 8: the 256 x 256 kernel for long prefill,
+       which needs n % 256 == 0, k >= 256 and grouped scales and otherwise leaves the call to the
+       128-column kernel), bits 20..21 wave quartets per workgroup (1 or 2). */
 };
 
 int uniql_abi_version(void);

@@ -20,6 +20,10 @@ size_t tile_part_bytes(int m, int n, int k, unsigned tune);
 bool tile_shape_ok(int m, int n, int k, int64_t ldx, unsigned tune);
 int pad_rows_launch(const void* A, int64_t lda, int k_in, void* dst, int k, int m, hipStream_t stream);
 size_t tile_accum_bytes(int m, int n, int k, unsigned tune = 0);
+int wide_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, const Epilogue& epi, int m, int n,
+                int k, int groups, hipStream_t stream);
+bool wide_shape_ok(int m, int n, int k, int groups, int64_t ldx);
+bool wide_preferred(int m, int n, int k, unsigned tune);
 int dequant_launch(const void* B, const void* S, void* W, uint8_t* codes, int n, int k, int groups,
                    hipStream_t stream);
 int embedding_launch(const int64_t* ids, int64_t ntokens, const void* weight, const void* scales, void* out,
@@ -120,6 +124,8 @@ int uniql_w4a16_linear_workspace(int m, int n, int k, int k_in, int had_block, u
     if (m == 0) return UNIQL_OK;
     const bool use_stream = takes_stream_kernel(m, flags);
     const unsigned tune = flags >> 8;
+    // (the 256 x 256 kernel needs neither buffer; the sizes are the 128 x 128 kernel's, which takes
+    // the call when the scales are per column)
     *accum_bytes = round256(use_stream ? stream_accum_bytes(m, n, k) : tile_accum_bytes(m, n, k, tune));
     // a strided input ahead of a separate rotation is compacted into the copy as well: count it
     const size_t act = had_block != 0 && fused_rotation(m, k, k_in, had_block, use_stream, flags) == 0
@@ -182,7 +188,10 @@ static int linear_impl(const void* A, int64_t lda, int k_in, const void* B, cons
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const bool use_stream = takes_stream_kernel(m, flags);
     const unsigned tune = flags >> 8;  // tuning fields, see the header
-    const size_t need_accum = round256(use_stream ? stream_accum_bytes(m, n, k) : tile_accum_bytes(m, n, k, tune));
+    // large M: the 256 x 256 kernel where it is the faster one and can take the call
+    const bool use_wide = !use_stream && wide_preferred(m, n, k, tune) && groups == k / 128;
+    const size_t need_accum =
+        round256(use_stream ? stream_accum_bytes(m, n, k) : use_wide ? 0 : tile_accum_bytes(m, n, k, tune));
     if (need_accum > 0 && (!accum || accum_bytes < need_accum)) return UNIQL_E_WORKSPACE;
 
     const void* Ain = A;
@@ -195,11 +204,13 @@ static int linear_impl(const void* A, int64_t lda, int k_in, const void* B, cons
     const bool pad_first = rotate_first ? (k_in != k || lda != k) : (k_in != k && !use_stream);
     // temp: the copy of the activations, then the tiled kernel's partial tiles when it splits K
     const size_t act_bytes = (rotate_first || pad_first) ? round256((size_t)m * k * sizeof(half_t)) : 0;
-    const size_t part_bytes = use_stream ? 0 : tile_part_bytes(m, n, k, tune);
+    const size_t part_bytes = (use_stream || use_wide) ? 0 : tile_part_bytes(m, n, k, tune);
     if (act_bytes + part_bytes > 0 && (!temp || temp_bytes < act_bytes + part_bytes)) return UNIQL_E_WORKSPACE;
     void* part = part_bytes ? reinterpret_cast<char*>(temp) + act_bytes : nullptr;
     // last check before the first kernel is enqueued: whether the tiled kernel can take the shape
-    if (!use_stream && !tile_shape_ok(m, n, k, (rotate_first || pad_first) ? (int64_t)k : lda, tune)) return UNIQL_E_SHAPE;
+    if (use_wide && !wide_shape_ok(m, n, k, groups, (rotate_first || pad_first) ? (int64_t)k : lda)) return UNIQL_E_SHAPE;
+    if (!use_stream && !use_wide && !tile_shape_ok(m, n, k, (rotate_first || pad_first) ? (int64_t)k : lda, tune))
+        return UNIQL_E_SHAPE;
     if (use_stream && !stream_shape_ok(k, (rotate_first || pad_first) ? (int64_t)k : lda)) return UNIQL_E_SHAPE;
     if (check_only) return UNIQL_OK;
     if (pad_first) {
@@ -228,6 +239,7 @@ static int linear_impl(const void* A, int64_t lda, int k_in, const void* B, cons
     epi.vec_ok = (!transpose && ldd % 8 == 0 && aligned16(D)) ? 1 : 0;
     if (use_stream)
         return stream_launch(Ain, ld, k_valid, B, S, D, epi, accum, m, n, k, groups, had_mode, had_scale, tune, st);
+    if (use_wide) return wide_launch(Ain, ld, B, S, D, epi, m, n, k, groups, st);
     return tile_launch(Ain, ld, B, S, D, epi, accum, accum_bytes, part, part_bytes, m, n, k, groups, tune, st);
 }
 

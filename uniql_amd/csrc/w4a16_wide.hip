@@ -1,0 +1,480 @@
+// Wide-tile W4A16 kernel for large M (long prefill): D[M,N] = X[M,K] . dequant(B)[K,N].
+//
+// A workgroup of four wavefronts owns a 256 x 256 output tile; wave (wm, wn) owns the 128 x 128
+// quarter (rows 128 wm.., columns 128 wn..) as 4 x 4 accumulators of v_mfma_f32_32x32x16_f16 and
+// keeps it for the whole of K, so there is no exchange of partial tiles at the end.  K advances in
+// blocks of 32 (two packed rows).  Per block
+//   * the X tile (256 rows x 32 K, 16 KiB) travels global -> LDS with global_load_lds_dwordx4,
+//   * the block's codes (2 packed rows x 256 columns, 4 KiB) and its scales travel the same way,
+//   * every weight of the block is expanded to the reference's fp16 value (code - 8) * scale ONCE
+//     per workgroup (one thread: the 32 codes of two columns x 16 K) and written to LDS as fp16,
+//     16 KiB, in MFMA operand order,
+//   * each wave reads 4 weight operands and 4 activation operands (16 bytes per lane each) per
+//     16 K and issues 16 MFMAs on them.
+// Against the 128 x 128 tiles of w4a16_tile_kernel (whose four waves split K and expand their own
+// weights) a weight is expanded once per 256 rows instead of once per 128, an X element is loaded
+// once per 256 columns instead of once per 128, and the weights no longer pass through the vector
+// ALU of the wave that multiplies them.  The price is the 256 x 256 granularity: the kernel is
+// chosen only where the grid still fills the chip (see wide_preferred).
+//
+// LDS operand layout (both tiles): element (x, k) of a block, x a row of X or a column of B, lives
+// in 16-byte unit 4 x + ((k / 8) ^ sw(x)), sw(x) = ((x >> 2) ^ (x >> 4)) & 3.  An MFMA operand read
+// (32 consecutive x, one K eighth per half-wave) then sweeps all 64 banks in every group of 16
+// lanes, and so do the 16-byte writes of the expansion (16 lanes: 4 column groups x 4 columns).
+//
+// Pipeline.  Rings: X blocks 4 slots, codes 4 slots, scales 3 slots (one per K group), expanded
+// weights 2 buffers.  Iteration kb multiplies block kb; meanwhile it expands the codes of block
+// kb+1 (fetched from LDS into registers during iteration kb-1) into the other weight buffer and,
+// after the one barrier of the iteration, reads the first operands of block kb+1, fetches the
+// codes of block kb+2 and issues the loads of X block kb+4 and of the codes of block kb+5 (into
+// slots everybody has finished reading before that barrier).  The loop is unrolled four times
+// (one K group), so every ring slot and with it every LDS address is a constant, and the scales
+// are loaded and fetched once per group.  A wave that has a SIMD to itself issues one instruction
+// every four clocks, whatever the instruction: the matrix pipe (32 clocks per MFMA) stays busy
+// only while the loop needs fewer than eight instructions per MFMA, so the instruction count is
+// what the code is written for.  vmcnt is counted by hand: an iteration issues five loads per
+// wave (four X pieces, then the codes), the first iteration of a group a sixth in front (scales),
+// and nothing else uses the counter inside the loop.  The last group runs a copy of the loop
+// body that issues no loads.
+#include <atomic>
+
+#include "common.hpp"
+
+#ifndef WIDE_ABL
+#define WIDE_ABL 0
+#endif
+
+namespace uniql {
+
+struct WideArgs {
+    const u32x4* B;
+    const half_t* S;
+    const half_t* X;
+    void* D;
+    int64_t ldx;
+    int M, N, K;
+    int mblocks;  // ceil(M / 256)
+    Epilogue epi;
+};
+
+typedef const __attribute__((address_space(1))) void* wide_gptr_t;
+typedef __attribute__((address_space(3))) void* wide_lptr_t;
+typedef uint32_t wide_u32x2 __attribute__((ext_vector_type(2)));
+
+// s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding)
+#define UNIQL_WIDE_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
+// s_waitcnt lgkmcnt(0) with the other counters left alone
+#define UNIQL_WIDE_WAIT_LGKM0() __builtin_amdgcn_s_waitcnt(0xC07F)
+
+constexpr int kWideXBytes = 256 * 64;   // one X block: 256 rows x 32 K x 2 bytes
+constexpr int kWideCBytes = 4096;       // one block of codes: 4 waves x 1 KiB
+constexpr int kWideSBytes = 4096;       // one group's scales: 4 waves x 1 KiB (256 bytes used per wave)
+constexpr int kWideWBytes = 256 * 64;   // one block of expanded weights: 256 columns x 32 K x 2 bytes
+constexpr int kWideXBase = 0;
+constexpr int kWideCBase = kWideXBase + 4 * kWideXBytes;
+constexpr int kWideSBase = kWideCBase + 4 * kWideCBytes;
+constexpr int kWideWBase = kWideSBase + 3 * kWideSBytes;
+constexpr int kWideLdsBytes = kWideWBase + 2 * kWideWBytes;  // 126976
+
+__device__ __forceinline__ int wide_sw(int x) { return ((x >> 2) ^ (x >> 4)) & 3; }
+
+template <int V>
+struct WideInt {
+    static constexpr int value = V;
+};
+
+template <bool EXT>
+__global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
+    char* const ldsb = reinterpret_cast<char*>(lds);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int w = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm = w >> 1, wn = w & 1;
+
+    // the M blocks of one column block are neighbours in launch order: they run together and the
+    // column block's codes are fetched from memory once
+    const int mblock = blockIdx.x % a.mblocks;
+    const int nblock = blockIdx.x / a.mblocks;
+    const int m0 = mblock * 256, n0 = nblock * 256;
+    const int ngroups = a.K >> 7;
+    const int N4 = a.N >> 1;  // 16-byte pieces per packed row
+
+    // ---- loads -------------------------------------------------------------------------
+    // Every load is "uniform 64-bit pointer + 32-bit lane offset" (the instruction's scalar-base
+    // form: no vector instruction for the address) into "constant + wave offset" of LDS.
+    // X: wave w brings rows 64 w .. 64 w + 63, 16 rows per operation; lane l lands in unit l of
+    // the operation's KiB, i.e. row l / 4, position l % 4, and fetches the K eighth that belongs
+    // there.  Rows past M re-read the last row (never stored).
+    uint32_t xsrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int row = 64 * w + 16 * i + (lane >> 2);
+        const int c = (lane & 3) ^ wide_sw(row);
+        const int rc = m0 + row < a.M ? row : a.M - 1 - m0;
+        xsrc[i] = (uint32_t)(((size_t)rc * a.ldx + 8 * c) * sizeof(half_t));
+    }
+    // codes: wave w brings packed row w / 2 of the block, column chunks 2 (w % 2), 2 (w % 2) + 1
+    // of the tile: one contiguous KiB, which the same wave expands
+    const uint32_t c_lane = 16u * lane;
+    // scales of the same 128 columns: lanes 0..15 fetch the 256 bytes, the others repeat them
+    const uint32_t s_lane = 16u * (lane & 15);
+    const size_t c_block_bytes = (size_t)2 * N4 * 16, s_group_bytes = (size_t)a.N * sizeof(half_t);
+    // the next block / group to request: running pointers, advanced after use
+    const char* x_next = reinterpret_cast<const char*>(a.X + (size_t)m0 * a.ldx);
+    const char* c_next = reinterpret_cast<const char*>(a.B + (size_t)(w >> 1) * N4 + (size_t)(n0 / 64 + 2 * (w & 1)) * 32);
+    const char* s_next = reinterpret_cast<const char*>(a.S + n0 + 128 * (w & 1));
+    const int wave_x = w * 4096, wave_kib = w * 1024;  // the wave's share of an X slot / of a codes or scales slot
+
+    auto load_x = [&](int slot, int i) __attribute__((always_inline)) {
+        const char* base = x_next;
+        uint32_t off = xsrc[i];
+        asm volatile("" : "+s"(base), "+v"(off));
+        __builtin_amdgcn_global_load_lds((wide_gptr_t)(base + off),
+                                         (wide_lptr_t)(ldsb + kWideXBase + slot * kWideXBytes + i * 1024 + wave_x), 16, 0, 0);
+    };
+    auto load_c = [&](int slot) __attribute__((always_inline)) {
+        const char* base = c_next;
+        uint32_t off = c_lane;
+        asm volatile("" : "+s"(base), "+v"(off));
+        __builtin_amdgcn_global_load_lds((wide_gptr_t)(base + off),
+                                         (wide_lptr_t)(ldsb + kWideCBase + slot * kWideCBytes + wave_kib), 16, 0, 0);
+    };
+    auto load_s = [&](int slot_bytes) __attribute__((always_inline)) {  // slot_bytes: uniform, 0 / 4096 / 8192
+        const char* base = s_next;
+        uint32_t off = s_lane;
+        asm volatile("" : "+s"(base), "+v"(off));
+        __builtin_amdgcn_global_load_lds((wide_gptr_t)(base + off),
+                                         (wide_lptr_t)(ldsb + kWideSBase + slot_bytes + wave_kib), 16, 0, 0);
+    };
+
+    // ---- expansion ---------------------------------------------------------------------
+    // Lane (cl, c8, j) of wave w takes the four words q = 0..3 at 128 cl + 16 c8 + 4 q + j of the
+    // wave's KiB: codes of columns 16 j + 8 blk + c8 (blk = 0, 1) of chunk 2 wn + cl, K values
+    // 8 hi + 2 q + lo of packed row w / 2.  Per (blk, hi) that is one 16-byte operand piece
+    // (eight consecutive K of one column).
+    const int cl = lane >> 5, c8 = (lane >> 2) & 7, j = lane & 3;
+    const int code_off = kWideCBase + wave_kib + 4 * (128 * cl + 16 * c8 + j);    // + slot * kWideCBytes + 16 q
+    const int scale_off = kWideSBase + wave_kib + 4 * (32 * cl + 4 * c8 + j);     // + slot bytes: halves (blk = 0, 1) at 64 cl + 8 c8 + 2 j
+    int wdst[2][2];  // byte offsets of the four pieces in weight buffer 0
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+        for (int hi = 0; hi < 2; ++hi) {
+            const int col = 64 * (2 * wn + cl) + 16 * j + 8 * blk + c8;
+            const int c = 2 * (w >> 1) + hi;
+            wdst[blk][hi] = kWideWBase + 16 * (4 * col + (c ^ wide_sw(col)));
+        }
+    NibbleMagic magic;
+    magic.init();
+    // The expansion of a block in pieces, so that the loop can spread it between its MFMAs:
+    // expand_fetch reads the lane's four words, expand_begin(e) / expand_end(e) make two of the 32
+    // values (e = 8 blk + 4 hi + q: word q, column blk, K values 8 hi + 2 q + {0, 1}; begin: the
+    // exact code - 8, end: the rounding multiplication by the scale), expand_store(blk, hi) writes
+    // one finished operand piece.  begin and end of a piece sit in different slots of the loop: a
+    // packed instruction right behind the one it depends on costs an idle issue slot.
+    uint32_t word[4], piece[16];
+    h2 scale_pair = h2{(half_t)0.f, (half_t)0.f};
+    auto expand_fetch = [&](int cslot) __attribute__((always_inline)) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) word[q] = *reinterpret_cast<const uint32_t*>(ldsb + code_off + cslot * kWideCBytes + 16 * q);
+    };
+    auto scale_fetch = [&](int slot_bytes) __attribute__((always_inline)) {
+        scale_pair = bits_to_h2(*reinterpret_cast<const uint32_t*>(ldsb + scale_off + slot_bytes));
+    };
+    auto expand_begin = [&](int e) __attribute__((always_inline)) {
+        const int blk = e >> 3, hi = (e >> 2) & 1, q = e & 3;
+        const uint32_t qq = blk ? (word[q] >> 8) : word[q];
+        uint32_t bits = h2_to_bits(hi ? magic.pair_high(qq) : magic.pair_low(qq));
+        asm volatile("" : "+v"(bits));  // pins the step to the place in the schedule where it is asked for
+        piece[e] = bits;
+    };
+    auto expand_end = [&](int e) __attribute__((always_inline)) {
+        const int blk = e >> 3;
+        const h2 sv = blk ? h2{scale_pair.y, scale_pair.y} : h2{scale_pair.x, scale_pair.x};
+        uint32_t bits = h2_to_bits(bits_to_h2(piece[e]) * sv);
+        asm volatile("" : "+v"(bits));
+        piece[e] = bits;
+    };
+    auto expand_store = [&](int buf, int blk, int hi) __attribute__((always_inline)) {
+        const int e = 8 * blk + 4 * hi;
+        *reinterpret_cast<u32x4*>(ldsb + wdst[blk][hi] + buf * kWideWBytes) = u32x4{piece[e], piece[e + 1], piece[e + 2], piece[e + 3]};
+    };
+
+    // ---- MFMA operands -------------------------------------------------------------------
+    // Operand (t, s): x = 128 wq + 32 t + r (r = lane % 32), K eighth 2 s + h (h = lane / 32):
+    // unit 4 x + ((2 s + h) ^ sw(x)), and sw(x) = sw(r) ^ 2 (t % 2).  With
+    //   u0 = 4 r + (h ^ (sw(r) & 1)) + (sw(r) & 2),  u1 = u0 ^ 2
+    // the unit is 512 wq + 128 t + (s ^ t) % 2 ? u1 : u0.
+    const int r = lane & 31, h = lane >> 5;
+    const int swr = wide_sw(r);
+    const int u0 = 4 * r + (h ^ (swr & 1)) + (swr & 2);
+    int xrd[2], wrd[2];  // byte offsets in X slot 0 / weight buffer 0
+    xrd[0] = kWideXBase + 16 * (512 * wm + u0);
+    xrd[1] = kWideXBase + 16 * (512 * wm + (u0 ^ 2));
+    wrd[0] = kWideWBase + 16 * (512 * wn + u0);
+    wrd[1] = kWideWBase + 16 * (512 * wn + (u0 ^ 2));
+
+    f16 acc[4][4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+#pragma unroll
+        for (int nt = 0; nt < 4; ++nt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[mt][nt][v] = 0.f;
+
+    h8 xa[2][4], bw[2][4];
+    // the i-th of the eight operand reads of a half, in the order the MFMAs want them: the
+    // first weight operand, the four activation operands, the other three weight operands
+    auto read_operand = [&](int set, int xslot, int wbuf, int s, int i) __attribute__((always_inline)) {
+        if (i >= 1 && i <= 4) {
+            const int t = i - 1;
+            xa[set][t] = *reinterpret_cast<const h8*>(ldsb + xrd[(s ^ t) & 1] + xslot * kWideXBytes + 2048 * t);
+        } else {
+            const int t = i == 0 ? 0 : i - 4;
+            bw[set][t] = *reinterpret_cast<const h8*>(ldsb + wrd[(s ^ t) & 1] + wbuf * kWideWBytes + 2048 * t);
+        }
+    };
+
+    // ---- prologue: the loads iterations -4 .. -1 would have issued, block 0 expanded ---------
+    int s_issue_bytes = 0;  // scales ring slot (as a byte offset) of the next group to request
+    int s_fetch_bytes = 0;  //                                      of the next group to fetch
+    auto advance3 = [&](int& slot_bytes) __attribute__((always_inline)) {
+        slot_bytes = slot_bytes == 2 * kWideSBytes ? 0 : slot_bytes + kWideSBytes;
+    };
+    load_c(0);
+    c_next += c_block_bytes;
+    // (the kernel runs on at least two groups; s_next never points past the last one)
+    load_s(s_issue_bytes);
+    s_next += s_group_bytes;
+    advance3(s_issue_bytes);
+    load_s(s_issue_bytes);
+    if (ngroups > 2) s_next += s_group_bytes;
+    advance3(s_issue_bytes);
+#pragma unroll
+    for (int b = 0; b < 4; ++b) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) load_x(b, i);
+        x_next += 64;
+        if (b < 3) {
+            load_c(b + 1);
+            c_next += c_block_bytes;
+        }
+    }
+    UNIQL_WIDE_WAIT_VMCNT(14);  // all but the last fourteen: codes 0 and 1, both groups of scales, X block 0
+    __builtin_amdgcn_s_barrier();
+    expand_fetch(0);
+    scale_fetch(s_fetch_bytes);
+    advance3(s_fetch_bytes);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) expand_begin(e);
+#pragma unroll
+    for (int e = 0; e < 16; ++e) expand_end(e);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) expand_store(0, e >> 1, e & 1);
+    expand_fetch(1);
+    UNIQL_WIDE_WAIT_LGKM0();  // the words of block 0 are in registers: their slot may take block 4
+    load_c(0);
+    c_next += c_block_bytes;
+    __builtin_amdgcn_s_barrier();
+#pragma unroll
+    for (int i = 0; i < 8; ++i) read_operand(0, 0, 0, 0, i);
+
+    size_t c_step = c_block_bytes;  // how far the codes pointer moves after an iteration
+    // ---- one iteration; J = kb % 4 is a constant --------------------------------------------
+    // One MFMA per slot, issued first; what else a slot does (in the matrix pipe's shadow) is
+    // fixed by hand and closed by a scheduling barrier.
+    // kVm: how many loads may be outstanding at the barrier: those of the last two iterations
+    // (what iteration kb-3 asked for, X block kb+1 and the codes of block kb+2, has landed then).
+    auto iteration = [&](auto jc, auto tailc) __attribute__((always_inline)) {
+        constexpr int J = decltype(jc)::value;
+        constexpr bool kTail = decltype(tailc)::value != 0;
+        constexpr int kVm = kTail ? (J == 0 ? 10 : J == 1 ? 5 : 0) : (J == 1 || J == 2 ? 11 : 10);
+        constexpr int xslot = J, xslot_next = (J + 1) & 3, wbuf = J & 1, wbuf_next = (J + 1) & 1;
+        // first half: K values 0..15 of block kb with operand set 0.  Meanwhile the second
+        // half's operands are read and block kb+1 is expanded into the other weight buffer.
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int nt = i >> 2, mt = i & 3;
+            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bw[0][nt], xa[0][mt], acc[mt][nt], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+#if WIDE_ABL != 5 && WIDE_ABL != 7
+            if (i < 8) read_operand(1, xslot, wbuf, 1, i);
+#endif
+#if WIDE_ABL != 3 && WIDE_ABL != 7
+            expand_begin(i);
+            if (i > 0) expand_end(i - 1);
+#endif
+            if (i == 5) expand_store(wbuf_next, 0, 0);
+            if (i == 9) expand_store(wbuf_next, 0, 1);
+            if (i == 13) expand_store(wbuf_next, 1, 0);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        // second half: K values 16..31 with operand set 1.  At the barrier the expanded
+        // weights of block kb+1 are written and everybody has read what the loads issued behind
+        // the barrier will overwrite.  Then: the next block's first operands, the words of block
+        // kb+2 (and, where that block starts a group, the group's scales), this iteration's loads.
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int nt = i >> 2, mt = i & 3;
+            acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bw[1][nt], xa[1][mt], acc[mt][nt], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i == 0) expand_end(15);
+            if (i == 1) expand_store(wbuf_next, 1, 1);
+            if (i == 4) {
+#if WIDE_ABL != 2
+                UNIQL_WIDE_WAIT_LGKM0();
+                UNIQL_WIDE_WAIT_VMCNT(kVm);
+                __builtin_amdgcn_s_barrier();
+#endif
+            }
+#if WIDE_ABL != 5 && WIDE_ABL != 7
+            if (i >= 5 && i < 13) read_operand(0, xslot_next, wbuf_next, 0, i - 5);
+#endif
+            if (i == 13) {
+                expand_fetch((J + 2) & 3);
+                if (J == 2) {
+                    scale_fetch(s_fetch_bytes);
+                    advance3(s_fetch_bytes);
+                }
+            }
+            if (!kTail && WIDE_ABL != 4 && WIDE_ABL != 7) {
+                if (J == 0 && i == 5) {
+                    load_s(s_issue_bytes);
+                    advance3(s_issue_bytes);
+                }
+                if (i == 6) load_x(xslot, 0);
+                if (i == 8) load_x(xslot, 1);
+                if (i == 10) load_x(xslot, 2);
+                if (i == 12) load_x(xslot, 3);
+                if (i == 14) load_c((J + 1) & 3);
+                if (i == 15) {
+                    x_next += 64;
+                    c_next += c_step;
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    // groups 0 .. ngroups-2 request what lies four and five blocks ahead (the scales two groups
+    // ahead: the last such request asks for the last group again); the last group requests nothing
+    for (int g = 0; g < ngroups - 1; ++g) {
+        iteration(WideInt<0>{}, WideInt<0>{});
+        if (g + 3 < ngroups) s_next += s_group_bytes;
+        iteration(WideInt<1>{}, WideInt<0>{});
+        // block kb + 5 of the last two iterations before the last group does not exist: they ask
+        // for the last block again (into a slot nobody reads any more)
+        if (g + 2 == ngroups) c_step = 0;
+        iteration(WideInt<2>{}, WideInt<0>{});
+        iteration(WideInt<3>{}, WideInt<0>{});
+    }
+    iteration(WideInt<0>{}, WideInt<1>{});
+    iteration(WideInt<1>{}, WideInt<1>{});
+    iteration(WideInt<2>{}, WideInt<1>{});
+    iteration(WideInt<3>{}, WideInt<1>{});
+    UNIQL_WIDE_WAIT_VMCNT(0);
+
+    // ---- store: acc[mt][nt][4 q + i] on lane l is row 128 wm + 32 mt + l % 32, column
+    // 128 wn + 32 nt + 8 q + 4 (l / 32) + i of the tile (the weights are the MFMA's first operand)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) {
+        const int m = m0 + 128 * wm + 32 * mt + r;
+        const bool row_exists = m < a.M;
+        if (EXT && a.epi.gated) {  // uniform: columns c and c + 64 of the wave's strip are a (gate, up) pair
+#pragma unroll
+            for (int nt = 0; nt < 2; ++nt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v)
+                    if (row_exists)
+                        finish_store_gated(a.epi, a.D, m, (n0 + 128 * wn) / 2 + 32 * nt + 8 * (v >> 2) + 4 * h + (v & 3),
+                                           acc[mt][nt][v], acc[mt][nt + 2][v]);
+        } else {
+#pragma unroll
+            for (int nt = 0; nt < 4; ++nt) {
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int n = n0 + 128 * wn + 32 * nt + 8 * q + 4 * h;
+                    const f16& t = acc[mt][nt];
+                    if (!row_exists) {
+                    } else if constexpr (EXT) {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) finish_store(a.epi, a.D, m, n + i, t[4 * q + i]);
+                    } else if (a.epi.out_f32) {
+                        *reinterpret_cast<f4*>(reinterpret_cast<float*>(a.D) + (size_t)m * a.N + n) =
+                            f4{t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
+                    } else {
+                        const h2 p0 = h2{(half_t)t[4 * q], (half_t)t[4 * q + 1]};
+                        const h2 p1 = h2{(half_t)t[4 * q + 2], (half_t)t[4 * q + 3]};
+                        *reinterpret_cast<wide_u32x2*>(reinterpret_cast<half_t*>(a.D) + (size_t)m * a.N + n) =
+                            wide_u32x2{h2_to_bits(p0), h2_to_bits(p1)};
+                    }
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------
+// Whether wide_launch can take the call at all: grouped scales, whole 256-column blocks, at
+// least the pipeline's six blocks of K, 32-bit in-tile offsets of the X loads.
+bool wide_shape_ok(int m, int n, int k, int groups, int64_t ldx) {
+    return m > 0 && n % 256 == 0 && k % 128 == 0 && k >= 256 && groups == k / 128 && ldx < (1LL << 23) &&
+           (int64_t)(n / 256) * ((m + 255) / 256) <= 0x7fffffffLL;
+}
+
+// Whether the entry point sends a call of the tiled path here.  tune: the tiled kernel's fields;
+// 8 in its "row tiles of 32 per workgroup" field (bits 8..11) asks for this kernel, any other
+// non-zero value there for the 128 x 128 one.
+// Without a forced choice: measured on the Llama and Mamba2 shapes at 256 to 8192 rows, the
+// 256 x 256 tiles win (by 5 to 30 %) where their grid keeps the chip busy: the share of real
+// output in the tile slots of its rounds of 256 workgroups is at least 0.62.
+bool wide_preferred(int m, int n, int k, unsigned tune) {
+    if (m <= 0 || n % 256 != 0 || k % 128 != 0 || k < 256) return false;
+    const int mt = (int)((tune >> 8) & 0xfu);
+    if (mt != 0) return mt == 8;
+    if ((tune & 0xffu) != 0 || ((tune >> 12) & 3u) != 0) return false;  // forced K splits or quartets: the 128 x 128 kernel's
+    const int64_t tiles = (int64_t)(n / 256) * ((m + 255) / 256);
+    const int64_t rounds = (tiles + 255) / 256;
+    return (double)m * n / 65536.0 >= 0.62 * 256.0 * (double)rounds;
+}
+
+template <bool EXT>
+static hipError_t wide_launch_one(const WideArgs& a, int grid, hipStream_t stream) {
+    auto kern = &w4a16_wide_kernel<EXT>;
+    static std::atomic<unsigned long long> done{0};  // the attribute is set once per device
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return hipErrorInvalidDevice;
+    if (dev < 0 || dev >= 64 || !((done.load(std::memory_order_relaxed) >> dev) & 1ull)) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           kWideLdsBytes);
+        if (e != hipSuccess) return e;
+        if (dev >= 0 && dev < 64) done.fetch_or(1ull << dev, std::memory_order_relaxed);
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), kWideLdsBytes, stream, a);
+    return hipGetLastError();
+}
+
+int wide_launch(const void* A, int64_t lda, const void* B, const void* S, void* D, const Epilogue& epi, int m, int n,
+                int k, int groups, hipStream_t stream) {
+    if (!wide_shape_ok(m, n, k, groups, lda)) return UNIQL_E_SHAPE;
+    WideArgs a;
+    a.B = reinterpret_cast<const u32x4*>(B);
+    a.S = reinterpret_cast<const half_t*>(S);
+    a.X = reinterpret_cast<const half_t*>(A);
+    a.D = D;
+    a.ldx = lda;
+    a.M = m;
+    a.N = n;
+    a.K = k;
+    a.mblocks = (m + 255) / 256;
+    a.epi = epi;
+    const int grid = (n / 256) * a.mblocks;
+    const bool ext = epi.gated || epi.bias || epi.residual || epi.relu2 || epi.transpose || epi.n_store != n ||
+                     epi.ldd != n;
+    const hipError_t e = ext ? wide_launch_one<true>(a, grid, stream) : wide_launch_one<false>(a, grid, stream);
+    return e == hipSuccess ? UNIQL_OK : UNIQL_E_LAUNCH;
+}
+
+}  // namespace uniql
