@@ -1,0 +1,173 @@
+"""GPU parity of the 256 x 256 tile kernel (long prefill), forced through the tuning field of the
+flags, against the oracle and against the 128-column kernel on the same calls."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import uniql_oracle as O
+from tests.helpers import check_layer_output, make_linear_problem, reference_product, to_gpu, workspace_for
+from tests.test_gpu_fused import assert_close16, deinterleave, gated_problem
+
+pytestmark = pytest.mark.gpu
+
+WIDE = 8 << 16      # "row tiles of 32 per workgroup" = 8: the 256 x 256 kernel
+NARROW = 4 << 16    # the 128-column kernel with 128-row tiles
+
+
+def run(p, dev, **kw):
+    from uniql_amd import ops
+    x, b, s = to_gpu(p, dev)
+    y = ops.w4a16_gemm_ex(x, b, s, workspace_for(p["n"], dev), p["m"], p["n"], p["k"], **kw)
+    torch.cuda.synchronize()
+    return y.cpu().numpy()
+
+
+@pytest.mark.parametrize("m,k,n", [(256, 256, 256), (300, 512, 512), (257, 384, 768), (1000, 1024, 768), (513, 4096, 512),
+                                   (17, 256, 256), (700, 1408, 256)])
+def test_wide_kernel_against_the_oracle(gpu, m, k, n):
+    """ragged M (rows past M inside the last tile), the shortest K (two groups), K groups that are
+    not a power of two; fp32 output against the float64 product, fp16 output = its rounding"""
+    p = make_linear_problem(m, k, n, seed=m + k + n)
+    ref = reference_product(p, exact=True)
+    y32 = run(p, gpu, out_f32=True, flags=WIDE)
+    assert np.abs(y32 - ref).max() < 2e-4, np.abs(y32 - ref).max()
+    y16 = run(p, gpu, flags=WIDE)
+    assert np.array_equal(y16.view(np.uint16), y32.astype(np.float16).view(np.uint16))
+    check_layer_output(y16, ref)
+    assert np.array_equal(run(p, gpu, flags=WIDE), y16)  # same result from run to run
+    # the 128-column kernel adds the same products in another order
+    other = run(p, gpu, out_f32=True, flags=NARROW)
+    assert np.abs(other - y32).max() < 1e-4
+
+
+def test_wide_kernel_long_k(gpu):
+    p = make_linear_problem(260, 14336, 256, seed=5)
+    ref = reference_product(p, exact=True)
+    y32 = run(p, gpu, out_f32=True, flags=WIDE)
+    assert np.abs(y32 - ref).max() < 1e-4
+    check_layer_output(run(p, gpu, flags=WIDE), ref)
+
+
+def test_wide_kernel_strided_rows(gpu):
+    from uniql_amd import ops
+    p = make_linear_problem(300, 512, 256, seed=9)
+    x, b, s = to_gpu(p, gpu)
+    big = torch.zeros(300, 1024 + 8, dtype=torch.float16, device=gpu)
+    big[:, 8:8 + 512] = x
+    y = ops.w4a16_gemm_ex(big[:, 8:8 + 512], b, s, workspace_for(256, gpu), 300, 256, 512, flags=WIDE)
+    want = ops.w4a16_gemm_ex(x, b, s, workspace_for(256, gpu), 300, 256, 512, flags=WIDE)
+    assert torch.equal(y, want)
+    check_layer_output(y.cpu().numpy(), reference_product(p))
+
+
+@pytest.mark.parametrize("m", [256, 300])
+@pytest.mark.parametrize("k,n,n_out", [(256, 256, 200), (640, 512, 512)])
+def test_wide_kernel_cut_bias_residual_relu2(gpu, m, k, n, n_out):
+    """the layer call's epilogues: bit-exact against the same kernel's plain product followed by
+    torch's fp16 operations"""
+    from uniql_amd import ops
+    p = make_linear_problem(m, k, n, seed=m + k)
+    x, b, s = to_gpu(p, gpu)
+    ws = workspace_for(n, gpu)
+    gen = torch.Generator().manual_seed(m + n)
+    bias = torch.randn(n_out, generator=gen).half().to(gpu)
+    res = torch.randn(m, n_out, generator=gen).half().to(gpu)
+    full = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k, flags=WIDE)
+    cut = ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, flags=WIDE)
+    assert torch.equal(cut, full[:, :n_out])
+    biased = ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, bias=bias, flags=WIDE)
+    assert torch.equal(biased, full[:, :n_out] + bias)
+    assert torch.equal(ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, bias=bias, residual=res, flags=WIDE),
+                       res + biased)
+    sq = ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, bias=bias, relu2=True, flags=WIDE)
+    assert torch.equal(sq, torch.relu(biased) ** 2)
+    y32 = ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, bias=bias, out_f32=True, flags=WIDE)
+    full32 = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k, out_f32=True, flags=WIDE)
+    assert torch.equal(y32, full32[:, :n_out] + bias.float())
+    # into a column range of a wider buffer
+    buf = torch.full((m, n_out + 40), 7.0, dtype=torch.float16, device=gpu)
+    ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, out=buf[:, 16:16 + n_out], flags=WIDE)
+    assert torch.equal(buf[:, 16:16 + n_out], cut)
+    assert bool((buf[:, :16] == 7).all()) and bool((buf[:, 16 + n_out:] == 7).all())
+
+
+@pytest.mark.parametrize("m", [256, 290])
+def test_wide_kernel_transposed_output(gpu, m):
+    from uniql_amd import ops
+    p = make_linear_problem(m, 256, 256, seed=m)
+    x, b, s = to_gpu(p, gpu)
+    ws = workspace_for(256, gpu)
+    plain = ops.w4a16_gemm_ex(x, b, s, ws, m, 256, 256, flags=WIDE)
+    t = ops.w4a16_gemm_ex(x, b, s, ws, m, 256, 256, transpose_out=True, flags=WIDE)
+    assert torch.equal(t[:, :m], plain.t())
+
+
+@pytest.mark.parametrize("m", [256, 300])
+@pytest.mark.parametrize("k,width,n_out", [(256, 128, 128), (512, 256, 200)])
+def test_wide_kernel_gated_pairs(gpu, m, k, width, n_out):
+    from uniql_amd import ops
+    g, u, w, s = gated_problem(m, k, width, seed=m + k)
+    x = torch.from_numpy(g["x"]).to(gpu)
+    w, s = w.to(gpu), s.to(gpu)
+    ws = workspace_for(2 * width, gpu)
+    both = ops.w4a16_gemm_ex(x, w, s, ws, m, 2 * width, k, flags=WIDE).cpu().numpy()
+    g16, u16 = deinterleave(both, width)
+    y = ops.w4a16_linear(x, w, s, ws, 2 * width, k, out_features=n_out, silu_mul=True, flags=WIDE)
+    assert y.shape == (m, n_out)
+    assert_close16(y.cpu().numpy(), O.mlp_gate_up(g16[:, :n_out], u16[:, :n_out]), ulps=2)
+    bias = torch.from_numpy(np.random.default_rng(m).standard_normal(2 * n_out).astype(np.float16)).to(gpu)
+    yb = ops.w4a16_linear(x, w, s, ws, 2 * width, k, out_features=n_out, silu_mul=True, bias=bias, flags=WIDE)
+    bn = bias.cpu().numpy().astype(np.float32)
+    gb = (g16[:, :n_out].astype(np.float32) + bn[:n_out]).astype(np.float16)
+    ub = (u16[:, :n_out].astype(np.float32) + bn[n_out:]).astype(np.float16)
+    assert_close16(yb.cpu().numpy(), O.mlp_gate_up(gb, ub), ulps=2)
+
+
+def test_wide_kernel_behind_a_rotation_and_a_short_input(gpu):
+    """the rotation and the zero padding of a short input run first, into the temporary buffer"""
+    from uniql_amd import ops
+    p = make_linear_problem(300, 512, 256, seed=31)
+    x, b, s = to_gpu(p, gpu)
+    ws = workspace_for(256, gpu)
+    for had in (128, 512):
+        got = ops.w4a16_gemm_ex(x, b, s, ws, 300, 256, 512, had_block=had, had_scale=had ** -0.5, flags=WIDE)
+        want = ops.w4a16_gemm_ex(ops.hadamard_blockwise(x, had ** -0.5, had), b, s, ws, 300, 256, 512, flags=WIDE)
+        assert torch.equal(got, want)
+    short = x[:, :456].contiguous()
+    padded = torch.zeros_like(x)
+    padded[:, :456] = short
+    assert torch.equal(ops.w4a16_linear(short, b, s, ws, 256, 512, flags=WIDE),
+                       ops.w4a16_gemm_ex(padded, b, s, ws, 300, 256, 512, flags=WIDE))
+
+
+def test_wide_request_falls_back_where_the_kernel_cannot_run(gpu):
+    """per-column scales, a width that is no multiple of 256, a single K group: the call is
+    served by the 128-column kernel"""
+    p = make_linear_problem(300, 384, 256, seed=3, per_column=True)
+    assert np.abs(run(p, gpu, out_f32=True, flags=WIDE) - reference_product(p, exact=True)).max() < 2e-4
+    p = make_linear_problem(300, 256, 384, seed=4)
+    assert np.abs(run(p, gpu, out_f32=True, flags=WIDE) - reference_product(p, exact=True)).max() < 2e-4
+    p = make_linear_problem(300, 128, 256, seed=5)
+    assert np.abs(run(p, gpu, out_f32=True, flags=WIDE) - reference_product(p, exact=True)).max() < 2e-4
+
+
+def test_wide_kernel_in_a_graph(gpu):
+    from uniql_amd import ops
+    p = make_linear_problem(512, 512, 512, seed=12)
+    x, b, s = to_gpu(p, gpu)
+    ws = workspace_for(512, gpu)
+    eager = ops.w4a16_gemm_ex(x, b, s, ws, 512, 512, 512, flags=WIDE)
+    out = torch.empty_like(eager)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops.w4a16_gemm_ex(x, b, s, ws, 512, 512, 512, flags=WIDE)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out.copy_(ops.w4a16_gemm_ex(x, b, s, ws, 512, 512, 512, flags=WIDE))
+    for _ in range(3):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)
