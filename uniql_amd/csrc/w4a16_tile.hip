@@ -63,6 +63,12 @@ struct TileArgs {
 typedef const __attribute__((address_space(1))) void* gptr_t;
 typedef __attribute__((address_space(3))) void* lptr_t;
 
+// 16 bytes per lane from a buffer (descriptor + lane offset + uniform offset) straight into LDS
+// (64 lanes fill one contiguous KiB at `dst`)
+__device__ __forceinline__ void buffer_to_lds16(__amdgpu_buffer_rsrc_t rsrc, uint32_t* dst, uint32_t lane_bytes, uint32_t uniform_bytes) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (lptr_t)dst, 16, lane_bytes, uniform_bytes, 0, 0);
+}
+
 // s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding)
 #define UNIQL_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
 
@@ -259,24 +265,30 @@ __global__ __launch_bounds__(256 * KW, 1) void w4a16_tile_kernel(const TileArgs 
     // The operations of a stage are spread between the MFMA blocks of the previous stage, so
     // the wave never sits behind a full address queue (the tile needs ~60% of the CU's
     // 64 B/clk vector-memory path).
+    // Every load is a buffer load into LDS: a descriptor (uniform base), a 32-bit lane offset that
+    // never changes and a uniform 32-bit offset that depends on the group, so that no vector
+    // instruction goes into an address (the host keeps the packed weights below 4 GiB).
+    constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
+    const __amdgpu_buffer_rsrc_t x_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(x_tile), 0, 0xffffffffu, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t w_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<u32x4*>(strip_w), 0, 0xffffffffu, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t s_rsrc = __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(strip_s), 0, 0xffffffffu, kRsrcFlags);
+    const uint32_t piece_bytes = 16u * piece_off, scale_lane_bytes = 16u * (uint32_t)dslot;
+    const uint32_t packed_row_bytes = 16u * (uint32_t)N4, scale_row_bytes = 2u * (uint32_t)scale_row_stride;
     auto issue_piece = [&](int g, int ring, int idx) __attribute__((always_inline)) {
         uint32_t* stage = lds + ring * L::kStageDwords;
         if (idx < kXOps) {
             uint32_t* xbuf = stage + (kXOps * 4 * w) * 64;  // this wave's X rows
-            const char* xg = reinterpret_cast<const char*>(x_tile + 128 * g);  // uniform
-            __builtin_amdgcn_global_load_lds((gptr_t)(xg + xsrc[idx]), (lptr_t)(xbuf + idx * 256), 16, 0, 0);
+            buffer_to_lds16(x_rsrc, xbuf + idx * 256, xsrc[idx], 256u * (uint32_t)g);
         } else if (idx < kXOps + 2) {
             uint32_t* bbuf = stage + L::kXDwords + w * 512 + (idx - kXOps) * 256;
-            const u32x4* rowp = strip_w + (size_t)(8 * g + 4 * (idx - kXOps)) * N4;  // uniform
-            __builtin_amdgcn_global_load_lds((gptr_t)(rowp + piece_off), (lptr_t)bbuf, 16, 0, 0);
+            buffer_to_lds16(w_rsrc, bbuf, piece_bytes, (uint32_t)(8 * g + 4 * (idx - kXOps)) * packed_row_bytes);
         } else {
             // scales of the group (row 0 in per-column mode, unused then)
             // all 64 lanes of all four waves take part (a predicated load would split the loop
             // body into several scheduling regions): every quarter-wave fetches the same 256
             // bytes, and the four waves write the same values to the same place
             uint32_t* sbuf = stage + L::kXDwords + L::kBDwords;
-            const half_t* ssrc = strip_s + (size_t)g * scale_row_stride;
-            __builtin_amdgcn_global_load_lds((gptr_t)(ssrc + 8 * dslot), (lptr_t)sbuf, 16, 0, 0);
+            buffer_to_lds16(s_rsrc, sbuf, scale_lane_bytes, (uint32_t)g * scale_row_bytes);
         }
     };
     auto issue_stage = [&](int g, int ring) __attribute__((always_inline)) {
@@ -662,13 +674,13 @@ static TilePlan tile_plan(int m, int n, int k, int splits_override, int mt_overr
     return p;
 }
 
-// Whether tile_launch can take the call: grid size, and the 32-bit in-tile offsets of the X loads
-// (128 rows of ldx elements, 2 bytes each, must stay below 2^32).  Checked by the entry point
+// Whether tile_launch can take the call: grid size, and the 32-bit offsets of the loads (128 rows of
+// ldx elements, 2 bytes each, and the packed weights must stay below 2^32 bytes).  Checked by the entry point
 // before anything is enqueued.
 bool tile_shape_ok(int m, int n, int k, int64_t ldx, unsigned tune) {
     const TilePlan plan = tile_plan_tuned(m, n, k, tune);
     const int64_t grid = (int64_t)(n / 128) * ceil_div_i(m, 32 * plan.mtiles) * plan.splits;
-    return grid <= 0x7fffffffLL && ldx < (1LL << 24);
+    return grid <= 0x7fffffffLL && ldx < (1LL << 24) && (int64_t)k * n / 2 < (1LL << 32);
 }
 
 template <int MT, bool EXT, int KW>

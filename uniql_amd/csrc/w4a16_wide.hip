@@ -18,9 +18,10 @@
 // chosen only where the grid still fills the chip (see wide_preferred).
 //
 // LDS operand layout (both tiles): element (x, k) of a block, x a row of X or a column of B, lives
-// in 16-byte unit 4 x + ((k / 8) ^ sw(x)), sw(x) = ((x >> 2) ^ (x >> 4)) & 3.  An MFMA operand read
-// (32 consecutive x, one K eighth per half-wave) then sweeps all 64 banks in every group of 16
-// lanes, and so do the 16-byte writes of the expansion (16 lanes: 4 column groups x 4 columns).
+// in 16-byte unit 4 x + ((k / 8) ^ sw(x)) with a two-bit XOR swizzle sw of the bits of x, chosen
+// so that neither an MFMA operand read (32 consecutive x, one K eighth per half-wave) nor a
+// 16-byte write of the expansion (lanes: 4 column groups x 8 columns x 2 chunks) meets a bank
+// conflict.
 //
 // Pipeline.  Rings: X blocks 4 slots, codes 4 slots, scales 3 slots (one per K group), expanded
 // weights 2 buffers.  Iteration kb multiplies block kb; meanwhile it expands the codes of block
@@ -66,17 +67,22 @@ typedef uint32_t wide_u32x2 __attribute__((ext_vector_type(2)));
 // s_waitcnt lgkmcnt(0) with the other counters left alone
 #define UNIQL_WIDE_WAIT_LGKM0() __builtin_amdgcn_s_waitcnt(0xC07F)
 
-constexpr int kWideXBytes = 256 * 64;   // one X block: 256 rows x 32 K x 2 bytes
+constexpr int kWideXBytes = 256 * 128;  // one X slot: 256 rows x 64 K (a pair of blocks) x 2 bytes
 constexpr int kWideCBytes = 4096;       // one block of codes: 4 waves x 1 KiB
 constexpr int kWideSBytes = 4096;       // one group's scales: 4 waves x 1 KiB (256 bytes used per wave)
 constexpr int kWideWBytes = 256 * 64;   // one block of expanded weights: 256 columns x 32 K x 2 bytes
 constexpr int kWideXBase = 0;
-constexpr int kWideCBase = kWideXBase + 4 * kWideXBytes;
+constexpr int kWideCBase = kWideXBase + 2 * kWideXBytes;
 constexpr int kWideSBase = kWideCBase + 4 * kWideCBytes;
 constexpr int kWideWBase = kWideSBase + 3 * kWideSBytes;
 constexpr int kWideLdsBytes = kWideWBase + 2 * kWideWBytes;  // 126976
 
-__device__ __forceinline__ int wide_sw(int x) { return ((x >> 2) ^ (x >> 4)) & 3; }
+// bit 0 = x2 ^ x4, bit 1 = x2 ^ x5: of the XOR swizzles of this form the one (with a few equals)
+// for which a probe of 16-byte LDS accesses showed no extra passes for either access pattern
+__device__ __forceinline__ int wide_sw(int x) { return (((x >> 2) ^ (x >> 4)) & 1) | ((((x >> 2) ^ (x >> 5)) & 1) << 1); }
+
+// X rows are 128 bytes (eight 16-byte chunks): chunk c of row x sits at position c ^ sw8(x)
+__device__ __forceinline__ int wide_sw8(int x) { return (x >> 1) & 7; }
 
 template <int V>
 struct WideInt {
@@ -102,16 +108,18 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
     const int N4 = a.N >> 1;  // 16-byte pieces per packed row
 
     // ---- loads -------------------------------------------------------------------------
-    // Every load is "uniform 64-bit pointer + 32-bit lane offset" (the instruction's scalar-base
-    // form: no vector instruction for the address) into "constant + wave offset" of LDS.
-    // X: wave w brings rows 64 w .. 64 w + 63, 16 rows per operation; lane l lands in unit l of
-    // the operation's KiB, i.e. row l / 4, position l % 4, and fetches the K eighth that belongs
-    // there.  Rows past M re-read the last row (never stored).
-    uint32_t xsrc[4];
+    // Every load is a buffer load into LDS: a descriptor (uniform base), a 32-bit lane offset that
+    // never changes, and a uniform 32-bit offset that advances with K.  No vector instruction and
+    // one scalar addition per advance go into addresses.
+    // X: wave w brings rows 64 w .. 64 w + 63 of a pair of blocks (64 K = whole 128-byte lines),
+    // 8 rows per operation; lane l lands in unit l of the operation's KiB, i.e. row l / 8,
+    // position l % 8, and fetches the K eighth that belongs there.  Rows past M re-read the last
+    // row (never stored).
+    uint32_t xsrc[8];
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int row = 64 * w + 16 * i + (lane >> 2);
-        const int c = (lane & 3) ^ wide_sw(row);
+    for (int i = 0; i < 8; ++i) {
+        const int row = 64 * w + 8 * i + (lane >> 3);
+        const int c = (lane & 7) ^ wide_sw8(row);
         const int rc = m0 + row < a.M ? row : a.M - 1 - m0;
         xsrc[i] = (uint32_t)(((size_t)rc * a.ldx + 8 * c) * sizeof(half_t));
     }
@@ -120,33 +128,29 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
     const uint32_t c_lane = 16u * lane;
     // scales of the same 128 columns: lanes 0..15 fetch the 256 bytes, the others repeat them
     const uint32_t s_lane = 16u * (lane & 15);
-    const size_t c_block_bytes = (size_t)2 * N4 * 16, s_group_bytes = (size_t)a.N * sizeof(half_t);
-    // the next block / group to request: running pointers, advanced after use
-    const char* x_next = reinterpret_cast<const char*>(a.X + (size_t)m0 * a.ldx);
-    const char* c_next = reinterpret_cast<const char*>(a.B + (size_t)(w >> 1) * N4 + (size_t)(n0 / 64 + 2 * (w & 1)) * 32);
-    const char* s_next = reinterpret_cast<const char*>(a.S + n0 + 128 * (w & 1));
-    const int wave_x = w * 4096, wave_kib = w * 1024;  // the wave's share of an X slot / of a codes or scales slot
+    const uint32_t c_block_bytes = 16u * (uint32_t)a.N, s_group_bytes = 2u * (uint32_t)a.N;
+    constexpr int kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
+    const __amdgpu_buffer_rsrc_t x_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(a.X + (size_t)m0 * a.ldx), 0, 0xffffffffu, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t c_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+        const_cast<u32x4*>(a.B + (size_t)(w >> 1) * N4 + (size_t)(n0 / 64 + 2 * (w & 1)) * 32), 0, 0xffffffffu, kRsrcFlags);
+    const __amdgpu_buffer_rsrc_t s_rsrc =
+        __builtin_amdgcn_make_buffer_rsrc(const_cast<half_t*>(a.S + n0 + 128 * (w & 1)), 0, 0xffffffffu, kRsrcFlags);
+    // the next pair of X blocks / block of codes / group of scales to request: byte offsets, advanced after use
+    uint32_t x_next = 0, c_next = 0, s_next = 0;
+    const int wave_x = w * 8192, wave_kib = w * 1024;  // the wave's share of an X slot / of a codes or scales slot
 
     auto load_x = [&](int slot, int i) __attribute__((always_inline)) {
-        const char* base = x_next;
-        uint32_t off = xsrc[i];
-        asm volatile("" : "+s"(base), "+v"(off));
-        __builtin_amdgcn_global_load_lds((wide_gptr_t)(base + off),
-                                         (wide_lptr_t)(ldsb + kWideXBase + slot * kWideXBytes + i * 1024 + wave_x), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(x_rsrc, (wide_lptr_t)(ldsb + kWideXBase + slot * kWideXBytes + i * 1024 + wave_x),
+                                                 16, xsrc[i], x_next, 0, 0);
     };
     auto load_c = [&](int slot) __attribute__((always_inline)) {
-        const char* base = c_next;
-        uint32_t off = c_lane;
-        asm volatile("" : "+s"(base), "+v"(off));
-        __builtin_amdgcn_global_load_lds((wide_gptr_t)(base + off),
-                                         (wide_lptr_t)(ldsb + kWideCBase + slot * kWideCBytes + wave_kib), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(c_rsrc, (wide_lptr_t)(ldsb + kWideCBase + slot * kWideCBytes + wave_kib), 16,
+                                                 c_lane, c_next, 0, 0);
     };
     auto load_s = [&](int slot_bytes) __attribute__((always_inline)) {  // slot_bytes: uniform, 0 / 4096 / 8192
-        const char* base = s_next;
-        uint32_t off = s_lane;
-        asm volatile("" : "+s"(base), "+v"(off));
-        __builtin_amdgcn_global_load_lds((wide_gptr_t)(base + off),
-                                         (wide_lptr_t)(ldsb + kWideSBase + slot_bytes + wave_kib), 16, 0, 0);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(s_rsrc, (wide_lptr_t)(ldsb + kWideSBase + slot_bytes + wave_kib), 16, s_lane,
+                                                 s_next, 0, 0);
     };
 
     // ---- expansion ---------------------------------------------------------------------
@@ -203,16 +207,17 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
     };
 
     // ---- MFMA operands -------------------------------------------------------------------
-    // Operand (t, s): x = 128 wq + 32 t + r (r = lane % 32), K eighth 2 s + h (h = lane / 32):
-    // unit 4 x + ((2 s + h) ^ sw(x)), and sw(x) = sw(r) ^ 2 (t % 2).  With
-    //   u0 = 4 r + (h ^ (sw(r) & 1)) + (sw(r) & 2),  u1 = u0 ^ 2
-    // the unit is 512 wq + 128 t + (s ^ t) % 2 ? u1 : u0.
+    // Operand t of K sixteenth s of a block: x = 128 wq + 32 t + r (r = lane % 32), K eighth
+    // 2 s + h of the block (h = lane / 32).
+    // Weights (64 bytes per column): unit 4 x + ((2 s + h) ^ sw(x)), and sw(x) = sw(r) ^ 2 (t % 2):
+    // with u0 = 4 r + (h ^ (sw(r) & 1)) + (sw(r) & 2) the unit is 512 wq + 128 t + ((s ^ t) % 2 ? u0 ^ 2 : u0).
+    // Activations (128 bytes per row, block b of the pair): unit 8 x + ((4 b + 2 s + h) ^ sw8(r)).
     const int r = lane & 31, h = lane >> 5;
     const int swr = wide_sw(r);
     const int u0 = 4 * r + (h ^ (swr & 1)) + (swr & 2);
-    int xrd[2], wrd[2];  // byte offsets in X slot 0 / weight buffer 0
-    xrd[0] = kWideXBase + 16 * (512 * wm + u0);
-    xrd[1] = kWideXBase + 16 * (512 * wm + (u0 ^ 2));
+    int xrd[4], wrd[2];  // byte offsets in X slot 0 (index 2 b + s) / weight buffer 0
+#pragma unroll
+    for (int c2 = 0; c2 < 4; ++c2) xrd[c2] = kWideXBase + 16 * (1024 * wm + 8 * r + ((2 * c2 + h) ^ wide_sw8(r)));
     wrd[0] = kWideWBase + 16 * (512 * wn + u0);
     wrd[1] = kWideWBase + 16 * (512 * wn + (u0 ^ 2));
 
@@ -227,23 +232,26 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
     h8 xa[2][4], bw[2][4];
     // the i-th of the eight operand reads of a half, in the order the MFMAs want them: the
     // first weight operand, the four activation operands, the other three weight operands
-    auto read_operand = [&](int set, int xslot, int wbuf, int s, int i) __attribute__((always_inline)) {
+    // kblock: the block's number modulo 4 (its pair's X slot is kblock / 2, its half of the pair kblock % 2)
+    auto read_operand = [&](int set, int kblock, int wbuf, int s, int i) __attribute__((always_inline)) {
         if (i >= 1 && i <= 4) {
             const int t = i - 1;
-            xa[set][t] = *reinterpret_cast<const h8*>(ldsb + xrd[(s ^ t) & 1] + xslot * kWideXBytes + 2048 * t);
+            xa[set][t] = *reinterpret_cast<const h8*>(ldsb + xrd[2 * (kblock & 1) + s] + (kblock >> 1) * kWideXBytes + 4096 * t);
         } else {
             const int t = i == 0 ? 0 : i - 4;
             bw[set][t] = *reinterpret_cast<const h8*>(ldsb + wrd[(s ^ t) & 1] + wbuf * kWideWBytes + 2048 * t);
         }
     };
 
-    // ---- prologue: the loads iterations -4 .. -1 would have issued, block 0 expanded ---------
+    // ---- prologue: the loads the iterations before the first would have issued, block 0 expanded ---
     int s_issue_bytes = 0;  // scales ring slot (as a byte offset) of the next group to request
     int s_fetch_bytes = 0;  //                                      of the next group to fetch
     auto advance3 = [&](int& slot_bytes) __attribute__((always_inline)) {
         slot_bytes = slot_bytes == 2 * kWideSBytes ? 0 : slot_bytes + kWideSBytes;
     };
     load_c(0);
+    c_next += c_block_bytes;
+    load_c(1);
     c_next += c_block_bytes;
     // (the kernel runs on at least two groups; s_next never points past the last one)
     load_s(s_issue_bytes);
@@ -253,16 +261,17 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
     if (ngroups > 2) s_next += s_group_bytes;
     advance3(s_issue_bytes);
 #pragma unroll
-    for (int b = 0; b < 4; ++b) {
+    for (int i = 0; i < 4; ++i) load_x(0, i);
+    load_c(2);
+    c_next += c_block_bytes;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) load_x(b, i);
-        x_next += 64;
-        if (b < 3) {
-            load_c(b + 1);
-            c_next += c_block_bytes;
-        }
-    }
-    UNIQL_WIDE_WAIT_VMCNT(14);  // all but the last fourteen: codes 0 and 1, both groups of scales, X block 0
+    for (int i = 4; i < 8; ++i) load_x(0, i);
+    x_next += 128;
+    load_c(3);
+    c_next += c_block_bytes;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) load_x(1, i);
+    UNIQL_WIDE_WAIT_VMCNT(5);  // all but the last five: codes 0..2, both groups of scales, the first pair of X blocks
     __builtin_amdgcn_s_barrier();
     expand_fetch(0);
     scale_fetch(s_fetch_bytes);
@@ -281,7 +290,7 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
 #pragma unroll
     for (int i = 0; i < 8; ++i) read_operand(0, 0, 0, 0, i);
 
-    size_t c_step = c_block_bytes;  // how far the codes pointer moves after an iteration
+    uint32_t c_step = c_block_bytes;  // how far the codes offset moves after an iteration
     // ---- one iteration; J = kb % 4 is a constant --------------------------------------------
     // One MFMA per slot, issued first; what else a slot does (in the matrix pipe's shadow) is
     // fixed by hand and closed by a scheduling barrier.
@@ -290,8 +299,8 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
     auto iteration = [&](auto jc, auto tailc) __attribute__((always_inline)) {
         constexpr int J = decltype(jc)::value;
         constexpr bool kTail = decltype(tailc)::value != 0;
-        constexpr int kVm = kTail ? (J == 0 ? 10 : J == 1 ? 5 : 0) : (J == 1 || J == 2 ? 11 : 10);
-        constexpr int xslot = J, xslot_next = (J + 1) & 3, wbuf = J & 1, wbuf_next = (J + 1) & 1;
+        constexpr int kVm = J == 0 ? 14 : kTail ? 0 : J == 1 ? 2 : J == 2 ? 15 : 1;
+        constexpr int wbuf = J & 1, wbuf_next = (J + 1) & 1;
         // first half: K values 0..15 of block kb with operand set 0.  Meanwhile the second
         // half's operands are read and block kb+1 is expanded into the other weight buffer.
 #pragma unroll
@@ -299,16 +308,25 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
             const int nt = i >> 2, mt = i & 3;
             acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bw[0][nt], xa[0][mt], acc[mt][nt], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-#if WIDE_ABL != 5 && WIDE_ABL != 7
-            if (i < 8) read_operand(1, xslot, wbuf, 1, i);
+#if WIDE_ABL != 5 && WIDE_ABL != 7 && WIDE_ABL != 12
+            if (i < 8) read_operand(1, J, wbuf, 1, i);
 #endif
-#if WIDE_ABL != 3 && WIDE_ABL != 7
+#if WIDE_ABL != 3 && WIDE_ABL != 7 && WIDE_ABL != 11
             expand_begin(i);
             if (i > 0) expand_end(i - 1);
 #endif
             if (i == 5) expand_store(wbuf_next, 0, 0);
             if (i == 9) expand_store(wbuf_next, 0, 1);
             if (i == 13) expand_store(wbuf_next, 1, 0);
+            // an even iteration requests the upper rows of the pair of X blocks whose lower rows the
+            // iteration before has requested (the last group's first iteration included)
+            if ((J & 1) == 0 && (!kTail || J == 0) && WIDE_ABL != 4 && WIDE_ABL != 7 && WIDE_ABL != 11 && WIDE_ABL != 12) {
+                if (i == 8) load_x(((J + 2) >> 1) & 1, 4);
+                if (i == 10) load_x(((J + 2) >> 1) & 1, 5);
+                if (i == 12) load_x(((J + 2) >> 1) & 1, 6);
+                if (i == 14) load_x(((J + 2) >> 1) & 1, 7);
+                if (i == 15) x_next += 128;
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
         // second half: K values 16..31 with operand set 1.  At the barrier the expanded
@@ -325,12 +343,16 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
             if (i == 4) {
 #if WIDE_ABL != 2
                 UNIQL_WIDE_WAIT_LGKM0();
+#if WIDE_ABL != 1
                 UNIQL_WIDE_WAIT_VMCNT(kVm);
+#endif
+#if WIDE_ABL != 10
                 __builtin_amdgcn_s_barrier();
 #endif
+#endif
             }
-#if WIDE_ABL != 5 && WIDE_ABL != 7
-            if (i >= 5 && i < 13) read_operand(0, xslot_next, wbuf_next, 0, i - 5);
+#if WIDE_ABL != 5 && WIDE_ABL != 7 && WIDE_ABL != 12
+            if (i >= 5 && i < 13) read_operand(0, (J + 1) & 3, wbuf_next, 0, i - 5);
 #endif
             if (i == 13) {
                 expand_fetch((J + 2) & 3);
@@ -339,20 +361,19 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
                     advance3(s_fetch_bytes);
                 }
             }
-            if (!kTail && WIDE_ABL != 4 && WIDE_ABL != 7) {
+            if (!kTail && WIDE_ABL != 4 && WIDE_ABL != 7 && WIDE_ABL != 11 && WIDE_ABL != 12) {
                 if (J == 0 && i == 5) {
                     load_s(s_issue_bytes);
                     advance3(s_issue_bytes);
                 }
-                if (i == 6) load_x(xslot, 0);
-                if (i == 8) load_x(xslot, 1);
-                if (i == 10) load_x(xslot, 2);
-                if (i == 12) load_x(xslot, 3);
-                if (i == 14) load_c((J + 1) & 3);
-                if (i == 15) {
-                    x_next += 64;
-                    c_next += c_step;
+                if ((J & 1) == 1) {  // the lower rows of the pair after next, into the slot this barrier has freed
+                    if (i == 6) load_x(((J + 3) >> 1) & 1, 0);
+                    if (i == 8) load_x(((J + 3) >> 1) & 1, 1);
+                    if (i == 10) load_x(((J + 3) >> 1) & 1, 2);
+                    if (i == 12) load_x(((J + 3) >> 1) & 1, 3);
                 }
+                if (i == 14) load_c((J + 1) & 3);
+                if (i == 15) c_next += c_step;
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -418,9 +439,11 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
 
 // ---------------------------------------------------------------------------------
 // Whether wide_launch can take the call at all: grouped scales, whole 256-column blocks, at
-// least the pipeline's six blocks of K, 32-bit in-tile offsets of the X loads.
+// least two K groups (the pipeline's prologue), 32-bit byte offsets into the X tile (256 rows of
+// ldx elements) and into the packed weights.
 bool wide_shape_ok(int m, int n, int k, int groups, int64_t ldx) {
-    return m > 0 && n % 256 == 0 && k % 128 == 0 && k >= 256 && groups == k / 128 && ldx < (1LL << 23) &&
+    return m > 0 && n % 256 == 0 && k % 128 == 0 && k >= 256 && groups == k / 128 &&
+           (255 * ldx + k) * 2 < (1LL << 32) && (int64_t)k * n / 2 < (1LL << 32) &&
            (int64_t)(n / 256) * ((m + 255) / 256) <= 0x7fffffffLL;
 }
 
