@@ -4,8 +4,10 @@
 // quarter (rows 128 wm.., columns 128 wn..) as 4 x 4 accumulators of v_mfma_f32_32x32x16_f16 and
 // keeps it for the whole of K, so there is no exchange of partial tiles at the end.  K advances in
 // blocks of 32 (two packed rows).  Per block
-//   * the X tile (256 rows x 32 K, 16 KiB) travels global -> LDS with global_load_lds_dwordx4,
-//   * the block's codes (2 packed rows x 256 columns, 4 KiB) and its scales travel the same way,
+//   * the X tile (256 rows x 32 K) travels global -> LDS as buffer loads into LDS, two blocks at a
+//     time (64 K = whole 128-byte lines of every row, 32 KiB),
+//   * the block's codes (2 packed rows x 256 columns, 4 KiB) travel the same way, the scales once
+//     per K group,
 //   * every weight of the block is expanded to the reference's fp16 value (code - 8) * scale ONCE
 //     per workgroup (one thread: the 32 codes of two columns x 16 K) and written to LDS as fp16,
 //     16 KiB, in MFMA operand order,
@@ -17,33 +19,30 @@
 // ALU of the wave that multiplies them.  The price is the 256 x 256 granularity: the kernel is
 // chosen only where the grid still fills the chip (see wide_preferred).
 //
-// LDS operand layout (both tiles): element (x, k) of a block, x a row of X or a column of B, lives
-// in 16-byte unit 4 x + ((k / 8) ^ sw(x)) with a two-bit XOR swizzle sw of the bits of x, chosen
-// so that neither an MFMA operand read (32 consecutive x, one K eighth per half-wave) nor a
-// 16-byte write of the expansion (lanes: 4 column groups x 8 columns x 2 chunks) meets a bank
-// conflict.
+// LDS operand layout.  Weights: element (column x, k) of a block lives in 16-byte unit
+// 4 x + ((k / 8) ^ sw(x)); activations: element (row x, k) of a pair of blocks in unit
+// 8 x + ((k / 8) ^ sw8(x)).  The XOR swizzles are chosen so that neither an MFMA operand read
+// (32 consecutive x, one K eighth per half-wave) nor a 16-byte write of the expansion meets a bank
+// conflict (checked with a probe of 16-byte LDS accesses on the hardware).
 //
-// Pipeline.  Rings: X blocks 4 slots, codes 4 slots, scales 3 slots (one per K group), expanded
-// weights 2 buffers.  Iteration kb multiplies block kb; meanwhile it expands the codes of block
-// kb+1 (fetched from LDS into registers during iteration kb-1) into the other weight buffer and,
-// after the one barrier of the iteration, reads the first operands of block kb+1, fetches the
-// codes of block kb+2 and issues the loads of X block kb+4 and of the codes of block kb+5 (into
-// slots everybody has finished reading before that barrier).  The loop is unrolled four times
-// (one K group), so every ring slot and with it every LDS address is a constant, and the scales
-// are loaded and fetched once per group.  A wave that has a SIMD to itself issues one instruction
+// Pipeline.  Rings: X two slots (a pair of blocks each), codes four slots, scales three slots (one
+// per K group), expanded weights two buffers.  Iteration kb multiplies block kb; meanwhile it
+// expands the codes of block kb+1 (fetched from LDS into registers during iteration kb-1) into
+// the other weight buffer and, after the one barrier of the iteration, reads the first operands
+// of block kb+1, fetches the codes of block kb+2 and requests the codes of block kb+5.  The X
+// blocks of pair p are requested in two halves: the lower rows behind the barrier of iteration
+// 2p-3 (which frees the slot), the upper rows during the first half of iteration 2p-2; they are
+// first read behind the barrier of iteration 2p-1.  The loop is unrolled four times (one K
+// group), so every ring slot and with it every LDS address is a constant, and the scales are
+// requested and fetched once per group.  A wave that has a SIMD to itself issues one instruction
 // every four clocks, whatever the instruction: the matrix pipe (32 clocks per MFMA) stays busy
 // only while the loop needs fewer than eight instructions per MFMA, so the instruction count is
-// what the code is written for.  vmcnt is counted by hand: an iteration issues five loads per
-// wave (four X pieces, then the codes), the first iteration of a group a sixth in front (scales),
-// and nothing else uses the counter inside the loop.  The last group runs a copy of the loop
-// body that issues no loads.
+// what the code is written for (about 4.6 per MFMA).  vmcnt is counted by hand: nothing but the
+// loop's own loads uses the counter, and their number and order per iteration are fixed.  The
+// last group runs a copy of the loop body that requests nothing but the last upper rows.
 #include <atomic>
 
 #include "common.hpp"
-
-#ifndef WIDE_ABL
-#define WIDE_ABL 0
-#endif
 
 namespace uniql {
 
@@ -58,7 +57,6 @@ struct WideArgs {
     Epilogue epi;
 };
 
-typedef const __attribute__((address_space(1))) void* wide_gptr_t;
 typedef __attribute__((address_space(3))) void* wide_lptr_t;
 typedef uint32_t wide_u32x2 __attribute__((ext_vector_type(2)));
 
@@ -294,8 +292,13 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
     // ---- one iteration; J = kb % 4 is a constant --------------------------------------------
     // One MFMA per slot, issued first; what else a slot does (in the matrix pipe's shadow) is
     // fixed by hand and closed by a scheduling barrier.
-    // kVm: how many loads may be outstanding at the barrier: those of the last two iterations
-    // (what iteration kb-3 asked for, X block kb+1 and the codes of block kb+2, has landed then).
+    // kVm: how many loads may still be outstanding at the barrier, i.e. how many were issued after
+    // the youngest one that must have landed.  Behind an odd iteration's barrier the first block
+    // of the next pair is read: its upper rows were the last request of the previous iteration's
+    // first half, followed only by that iteration's codes (and scales, in a group's first
+    // iteration).  Behind an even iteration's barrier the codes of block kb+2 are fetched: the
+    // last request of iteration kb-3, followed by the 5 (6) requests each of iterations kb-2 and
+    // kb-1 and the 4 of this iteration's first half.
     auto iteration = [&](auto jc, auto tailc) __attribute__((always_inline)) {
         constexpr int J = decltype(jc)::value;
         constexpr bool kTail = decltype(tailc)::value != 0;
@@ -308,19 +311,15 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
             const int nt = i >> 2, mt = i & 3;
             acc[mt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bw[0][nt], xa[0][mt], acc[mt][nt], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
-#if WIDE_ABL != 5 && WIDE_ABL != 7 && WIDE_ABL != 12
             if (i < 8) read_operand(1, J, wbuf, 1, i);
-#endif
-#if WIDE_ABL != 3 && WIDE_ABL != 7 && WIDE_ABL != 11
             expand_begin(i);
             if (i > 0) expand_end(i - 1);
-#endif
             if (i == 5) expand_store(wbuf_next, 0, 0);
             if (i == 9) expand_store(wbuf_next, 0, 1);
             if (i == 13) expand_store(wbuf_next, 1, 0);
             // an even iteration requests the upper rows of the pair of X blocks whose lower rows the
             // iteration before has requested (the last group's first iteration included)
-            if ((J & 1) == 0 && (!kTail || J == 0) && WIDE_ABL != 4 && WIDE_ABL != 7 && WIDE_ABL != 11 && WIDE_ABL != 12) {
+            if ((J & 1) == 0 && (!kTail || J == 0)) {
                 if (i == 8) load_x(((J + 2) >> 1) & 1, 4);
                 if (i == 10) load_x(((J + 2) >> 1) & 1, 5);
                 if (i == 12) load_x(((J + 2) >> 1) & 1, 6);
@@ -341,19 +340,11 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
             if (i == 0) expand_end(15);
             if (i == 1) expand_store(wbuf_next, 1, 1);
             if (i == 4) {
-#if WIDE_ABL != 2
                 UNIQL_WIDE_WAIT_LGKM0();
-#if WIDE_ABL != 1
                 UNIQL_WIDE_WAIT_VMCNT(kVm);
-#endif
-#if WIDE_ABL != 10
                 __builtin_amdgcn_s_barrier();
-#endif
-#endif
             }
-#if WIDE_ABL != 5 && WIDE_ABL != 7 && WIDE_ABL != 12
             if (i >= 5 && i < 13) read_operand(0, (J + 1) & 3, wbuf_next, 0, i - 5);
-#endif
             if (i == 13) {
                 expand_fetch((J + 2) & 3);
                 if (J == 2) {
@@ -361,7 +352,7 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
                     advance3(s_fetch_bytes);
                 }
             }
-            if (!kTail && WIDE_ABL != 4 && WIDE_ABL != 7 && WIDE_ABL != 11 && WIDE_ABL != 12) {
+            if (!kTail) {
                 if (J == 0 && i == 5) {
                     load_s(s_issue_bytes);
                     advance3(s_issue_bytes);
