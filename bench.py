@@ -15,7 +15,7 @@ that launch overhead is the GPU's, not Python's, and replay boundaries are rare.
 value = algorithmic bytes per step / time per step  (GB/s), algorithmic bytes of a
 linear = K N / 2 + (K/128) N 2 + M K 2 + M N 2.  The same JSON line carries, under
 "prefill_gemm_m1024", the other half of the metric: the four linears at M = 1024 through
-the tiled MFMA kernel (TFLOP/s = 2 M K N / time, against 2.5 PFLOP/s dense fp16).
+the tiled MFMA kernels (TFLOP/s = 2 M K N / time, against 2.5 PFLOP/s dense fp16).
 
 --sweep additionally prints (stderr) and writes (--sweep-json, default bench_sweep.json in the
 working directory) the per-shape tables: decode M in {1,2,4,8}, prefill M in {256,1024,4096},
@@ -459,7 +459,8 @@ def main():
         "unit": "TFLOP/s", "us_per_layer": round(tot_sec * 1e6, 2), "per_linear": per_shape,
         "roofline": {"bound": "mfma", "achieved": round(tot_flops / tot_sec / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
                      "unit": "TFLOP/s", "frac": round(tot_flops / tot_sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-                     "kernel": "w4a16_tile_kernel<MT> (MT = 4, or 2 for the 6144-wide qkv)"}}
+                     "kernel": "w4a16_wide_kernel (256 x 256 tiles) for gate_up, w4a16_tile_kernel<MT> (MT = 4, or 2 for the "
+                               "6144-wide qkv) for the other three"}}
     if args.sweep:
         sweep(dev, gen, args.sweep_json)
     if not args.no_cpu:

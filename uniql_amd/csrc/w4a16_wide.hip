@@ -82,6 +82,95 @@ __device__ __forceinline__ int wide_sw(int x) { return (((x >> 2) ^ (x >> 4)) & 
 // X rows are 128 bytes (eight 16-byte chunks): chunk c of row x sits at position c ^ sw8(x)
 __device__ __forceinline__ int wide_sw8(int x) { return (x >> 1) & 7; }
 
+// Four consecutive fp16 values from p: one 8-byte load where the address allows it.
+__device__ __forceinline__ void wide_load_four(const half_t* p, bool aligned8, float (&out)[4]) {
+    if (aligned8) {
+        const wide_u32x2 w = *reinterpret_cast<const wide_u32x2*>(p);
+        const h2 a = bits_to_h2(w.x), b = bits_to_h2(w.y);
+        out[0] = (float)a.x;
+        out[1] = (float)a.y;
+        out[2] = (float)b.x;
+        out[3] = (float)b.y;
+    } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) out[i] = (float)p[i];
+    }
+}
+
+// Four consecutive outputs of row m starting at column n0 (a multiple of 4): one 8- or 16-byte
+// store where the output's layout allows it, element stores otherwise.  The roundings are those of
+// finish_half / finish_half_gated; bias and residual come as 8-byte loads where they are aligned.
+__device__ __forceinline__ void wide_store_four(const Epilogue& e, void* D, int m, int n0, f4 v) {
+    if (e.vec_ok && n0 + 4 <= e.n_store) {
+        const size_t o = (size_t)m * e.ldd + n0;
+        if (e.out_f32 && !e.bias && !e.residual && !e.relu2) {
+            *reinterpret_cast<f4*>(reinterpret_cast<float*>(D) + o) = v;
+            return;
+        }
+        if (!e.out_f32) {
+            half_t y[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) y[i] = (half_t)v[i];
+            if (e.bias) {
+                float b[4];
+                wide_load_four(e.bias + n0, (reinterpret_cast<uintptr_t>(e.bias) & 7u) == 0, b);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) y[i] = (half_t)((float)y[i] + b[i]);
+            }
+            if (e.relu2) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float r = (float)y[i] > 0.f ? (float)y[i] : 0.f;
+                    y[i] = (half_t)(r * r);
+                }
+            }
+            if (e.residual) {
+                float r[4];
+                wide_load_four(e.residual + (size_t)m * e.ldr + n0,
+                               (reinterpret_cast<uintptr_t>(e.residual) & 7u) == 0 && (e.ldr & 3) == 0, r);
+#pragma unroll
+                for (int i = 0; i < 4; ++i) y[i] = (half_t)(r[i] + (float)y[i]);
+            }
+            *reinterpret_cast<wide_u32x2*>(reinterpret_cast<half_t*>(D) + o) =
+                wide_u32x2{h2_to_bits(h2{y[0], y[1]}), h2_to_bits(h2{y[2], y[3]})};
+            return;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) finish_store(e, D, m, n0 + i, v[i]);
+}
+__device__ __forceinline__ void wide_store_four_gated(const Epilogue& e, void* D, int m, int n0, f4 g, f4 u) {
+    if (e.vec_ok && !e.out_f32 && n0 + 4 <= e.n_store) {
+        half_t g16[4], u16[4], y[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            g16[i] = (half_t)g[i];
+            u16[i] = (half_t)u[i];
+        }
+        if (e.bias) {
+            float bg[4], bu[4];
+            const bool al = (reinterpret_cast<uintptr_t>(e.bias) & 7u) == 0;
+            wide_load_four(e.bias + n0, al, bg);
+            wide_load_four(e.bias + e.n_store + n0, al && (e.n_store & 3) == 0, bu);
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                g16[i] = (half_t)((float)g16[i] + bg[i]);
+                u16[i] = (half_t)((float)u16[i] + bu[i]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const half_t a16 = (half_t)silu_f32((float)g16[i]);
+            y[i] = (half_t)((float)a16 * (float)u16[i]);
+        }
+        *reinterpret_cast<wide_u32x2*>(reinterpret_cast<half_t*>(D) + (size_t)m * e.ldd + n0) =
+            wide_u32x2{h2_to_bits(h2{y[0], y[1]}), h2_to_bits(h2{y[2], y[3]})};
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) finish_store_gated(e, D, m, n0 + i, g[i], u[i]);
+}
+
 template <int V>
 struct WideInt {
     static constexpr int value = V;
@@ -389,43 +478,53 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
     UNIQL_WIDE_WAIT_VMCNT(0);
 
     // ---- store: acc[mt][nt][4 q + i] on lane l is row 128 wm + 32 mt + l % 32, column
-    // 128 wn + 32 nt + 8 q + 4 (l / 32) + i of the tile (the weights are the MFMA's first operand)
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) {
-        const int m = m0 + 128 * wm + 32 * mt + r;
-        const bool row_exists = m < a.M;
-        if (EXT && a.epi.gated) {  // uniform: columns c and c + 64 of the wave's strip are a (gate, up) pair
-#pragma unroll
-            for (int nt = 0; nt < 2; ++nt)
-#pragma unroll
-                for (int v = 0; v < 16; ++v)
-                    if (row_exists)
-                        finish_store_gated(a.epi, a.D, m, (n0 + 128 * wn) / 2 + 32 * nt + 8 * (v >> 2) + 4 * h + (v & 3),
-                                           acc[mt][nt][v], acc[mt][nt + 2][v]);
-        } else {
-#pragma unroll
-            for (int nt = 0; nt < 4; ++nt) {
-#pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const int n = n0 + 128 * wn + 32 * nt + 8 * q + 4 * h;
-                    const f16& t = acc[mt][nt];
-                    if (!row_exists) {
-                    } else if constexpr (EXT) {
-#pragma unroll
-                        for (int i = 0; i < 4; ++i) finish_store(a.epi, a.D, m, n + i, t[4 * q + i]);
-                    } else if (a.epi.out_f32) {
-                        *reinterpret_cast<f4*>(reinterpret_cast<float*>(a.D) + (size_t)m * a.N + n) =
-                            f4{t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
-                    } else {
-                        const h2 p0 = h2{(half_t)t[4 * q], (half_t)t[4 * q + 1]};
-                        const h2 p1 = h2{(half_t)t[4 * q + 2], (half_t)t[4 * q + 3]};
-                        *reinterpret_cast<wide_u32x2*>(reinterpret_cast<half_t*>(a.D) + (size_t)m * a.N + n) =
-                            wide_u32x2{h2_to_bits(p0), h2_to_bits(p1)};
+    // 128 wn + 32 nt + 8 q + 4 (l / 32) + i of the tile (the weights are the MFMA's first operand).
+    // The lane's coordinates are derived again behind the loop (the empty asm keeps the compiler
+    // from computing the store addresses in front of it, where they would cost registers the loop needs).
+    int lane_s = lane;
+    asm volatile("" : "+v"(lane_s));
+    const int rs = lane_s & 31, hs = lane_s >> 5;
+    // (written with constant indices throughout: a loop the compiler declines to unroll would
+    // index the accumulators at run time and so move them from registers to memory, for the whole kernel)
+    auto four_times = [&](auto&& f) __attribute__((always_inline)) {
+        f(WideInt<0>{});
+        f(WideInt<1>{});
+        f(WideInt<2>{});
+        f(WideInt<3>{});
+    };
+    const bool gated = EXT && a.epi.gated != 0;  // uniform: columns c and c + 64 of the wave's strip are a (gate, up) pair
+    four_times([&](auto mtc) __attribute__((always_inline)) {
+        constexpr int mt = decltype(mtc)::value;
+        const int m = m0 + 128 * wm + 32 * mt + rs;
+        if (m >= a.M) return;
+        four_times([&](auto ntc) __attribute__((always_inline)) {
+            constexpr int nt = decltype(ntc)::value;
+            four_times([&](auto qc) __attribute__((always_inline)) {
+                constexpr int q = decltype(qc)::value;
+                const f16& t = acc[mt][nt];
+                const f4 v = f4{t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
+                if (gated) {
+                    if constexpr (nt < 2) {
+                        const f16& up = acc[mt][nt + 2];
+                        wide_store_four_gated(a.epi, a.D, m, (n0 + 128 * wn) / 2 + 32 * nt + 8 * q + 4 * hs, v,
+                                              f4{up[4 * q], up[4 * q + 1], up[4 * q + 2], up[4 * q + 3]});
                     }
+                    return;
                 }
-            }
-        }
-    }
+                const int n = n0 + 128 * wn + 32 * nt + 8 * q + 4 * hs;
+                if constexpr (EXT) {
+                    wide_store_four(a.epi, a.D, m, n, v);
+                } else if (a.epi.out_f32) {
+                    *reinterpret_cast<f4*>(reinterpret_cast<float*>(a.D) + (size_t)m * a.N + n) = v;
+                } else {
+                    const h2 p0 = h2{(half_t)v[0], (half_t)v[1]};
+                    const h2 p1 = h2{(half_t)v[2], (half_t)v[3]};
+                    *reinterpret_cast<wide_u32x2*>(reinterpret_cast<half_t*>(a.D) + (size_t)m * a.N + n) =
+                        wide_u32x2{h2_to_bits(p0), h2_to_bits(p1)};
+                }
+            });
+        });
+    });
 }
 
 // ---------------------------------------------------------------------------------
