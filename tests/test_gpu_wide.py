@@ -151,6 +151,20 @@ def test_wide_request_falls_back_where_the_kernel_cannot_run(gpu):
     assert np.abs(run(p, gpu, out_f32=True, flags=WIDE) - reference_product(p, exact=True)).max() < 2e-4
 
 
+def test_wide_request_with_a_row_stride_beyond_its_offsets(gpu):
+    """256 rows of `lda` elements must fit 32-bit byte offsets; a larger stride (still fine for the
+    128-column kernel) is served by that kernel"""
+    from uniql_amd import ops
+    p = make_linear_problem(260, 256, 256, seed=17)
+    x, b, s = to_gpu(p, gpu)
+    lda = (1 << 23) + 8
+    big = torch.empty(260 * lda, dtype=torch.float16, device=gpu).view(260, lda)
+    big[:, :256] = x
+    y = ops.w4a16_gemm_ex(big[:, :256], b, s, workspace_for(256, gpu), 260, 256, 256, out_f32=True, flags=WIDE)
+    assert np.abs(y.cpu().numpy() - reference_product(p, exact=True)).max() < 2e-4
+    del big
+
+
 def test_wide_kernel_in_a_graph(gpu):
     from uniql_amd import ops
     p = make_linear_problem(512, 512, 512, seed=12)

@@ -188,11 +188,6 @@ static int linear_impl(const void* A, int64_t lda, int k_in, const void* B, cons
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
     const bool use_stream = takes_stream_kernel(m, flags);
     const unsigned tune = flags >> 8;  // tuning fields, see the header
-    // large M: the 256 x 256 kernel where it is the faster one and can take the call
-    const bool use_wide = !use_stream && wide_preferred(m, n, k, tune) && groups == k / 128;
-    const size_t need_accum =
-        round256(use_stream ? stream_accum_bytes(m, n, k) : use_wide ? 0 : tile_accum_bytes(m, n, k, tune));
-    if (need_accum > 0 && (!accum || accum_bytes < need_accum)) return UNIQL_E_WORKSPACE;
 
     const void* Ain = A;
     int64_t ld = lda;
@@ -202,16 +197,20 @@ static int linear_impl(const void* A, int64_t lda, int k_in, const void* B, cons
     // the transform kernel reads dense rows of k values: a strided or short input is first copied
     // (and zero-padded) into the temporary buffer, then rotated there in place
     const bool pad_first = rotate_first ? (k_in != k || lda != k) : (k_in != k && !use_stream);
+    const int64_t ld_kernel = (rotate_first || pad_first) ? (int64_t)k : lda;  // row stride the product kernel will see
+    // large M: the 256 x 256 kernel where it is the faster one and can take the call
+    const bool use_wide = !use_stream && wide_preferred(m, n, k, tune) && wide_shape_ok(m, n, k, groups, ld_kernel);
+    const size_t need_accum =
+        round256(use_stream ? stream_accum_bytes(m, n, k) : use_wide ? 0 : tile_accum_bytes(m, n, k, tune));
+    if (need_accum > 0 && (!accum || accum_bytes < need_accum)) return UNIQL_E_WORKSPACE;
     // temp: the copy of the activations, then the tiled kernel's partial tiles when it splits K
     const size_t act_bytes = (rotate_first || pad_first) ? round256((size_t)m * k * sizeof(half_t)) : 0;
     const size_t part_bytes = (use_stream || use_wide) ? 0 : tile_part_bytes(m, n, k, tune);
     if (act_bytes + part_bytes > 0 && (!temp || temp_bytes < act_bytes + part_bytes)) return UNIQL_E_WORKSPACE;
     void* part = part_bytes ? reinterpret_cast<char*>(temp) + act_bytes : nullptr;
     // last check before the first kernel is enqueued: whether the tiled kernel can take the shape
-    if (use_wide && !wide_shape_ok(m, n, k, groups, (rotate_first || pad_first) ? (int64_t)k : lda)) return UNIQL_E_SHAPE;
-    if (!use_stream && !use_wide && !tile_shape_ok(m, n, k, (rotate_first || pad_first) ? (int64_t)k : lda, tune))
-        return UNIQL_E_SHAPE;
-    if (use_stream && !stream_shape_ok(k, (rotate_first || pad_first) ? (int64_t)k : lda)) return UNIQL_E_SHAPE;
+    if (!use_stream && !use_wide && !tile_shape_ok(m, n, k, ld_kernel, tune)) return UNIQL_E_SHAPE;
+    if (use_stream && !stream_shape_ok(k, ld_kernel)) return UNIQL_E_SHAPE;
     if (check_only) return UNIQL_OK;
     if (pad_first) {
         const int e = pad_rows_launch(A, lda, k_in, temp, k, m, st);
