@@ -151,6 +151,20 @@ def test_wide_request_falls_back_where_the_kernel_cannot_run(gpu):
     assert np.abs(run(p, gpu, out_f32=True, flags=WIDE) - reference_product(p, exact=True)).max() < 2e-4
 
 
+def test_wide_kernel_output_at_an_odd_address(gpu):
+    """an output that is only 2-byte aligned takes the element-wise stores"""
+    from uniql_amd import ops
+    p = make_linear_problem(300, 256, 256, seed=23)
+    x, b, s = to_gpu(p, gpu)
+    ws = workspace_for(256, gpu)
+    want = ops.w4a16_linear(x, b, s, ws, 256, 256, flags=WIDE)
+    flat = torch.zeros(300 * 256 + 8, dtype=torch.float16, device=gpu)
+    out = flat[1:1 + 300 * 256].view(300, 256)
+    ops.w4a16_linear(x, b, s, ws, 256, 256, out=out, flags=WIDE)
+    assert torch.equal(out, want)
+    assert float(flat[0]) == 0 and float(flat[-1]) == 0
+
+
 def test_wide_request_with_a_row_stride_beyond_its_offsets(gpu):
     """256 rows of `lda` elements must fit 32-bit byte offsets; a larger stride (still fine for the
     128-column kernel) is served by that kernel"""

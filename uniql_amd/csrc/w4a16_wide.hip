@@ -584,8 +584,9 @@ int wide_launch(const void* A, int64_t lda, const void* B, const void* S, void* 
     a.mblocks = (m + 255) / 256;
     a.epi = epi;
     const int grid = (n / 256) * a.mblocks;
+    // (the plain instantiation stores 8 or 16 bytes at a time: it also needs an aligned D)
     const bool ext = epi.gated || epi.bias || epi.residual || epi.relu2 || epi.transpose || epi.n_store != n ||
-                     epi.ldd != n;
+                     epi.ldd != n || !epi.vec_ok;
     const hipError_t e = ext ? wide_launch_one<true>(a, grid, stream) : wide_launch_one<false>(a, grid, stream);
     return e == hipSuccess ? UNIQL_OK : UNIQL_E_LAUNCH;
 }
