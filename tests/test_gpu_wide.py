@@ -199,3 +199,49 @@ def test_wide_kernel_in_a_graph(gpu):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
+
+
+def test_wide_kernel_random_shapes(gpu):
+    """600 seeded cases (rows 1..1100, K 256..2432 and a few long ones, 1..4 column blocks, strided
+    rows, plain / cut + bias / residual / gated calls) against a float64 product of the bit-exact
+    dequantised weights on the GPU; the hand-counted load pipeline has no shape it may miss"""
+    from uniql_amd import ops
+    import bench
+    cache = {}
+    for seed in range(600):
+        rng = np.random.default_rng(seed)
+        gen = torch.Generator(device=gpu).manual_seed(seed)
+        k = 128 * int(rng.integers(2, 20)) if rng.integers(0, 6) else 128 * int(rng.integers(20, 120))
+        n = 256 * int(rng.integers(1, 5))
+        m = int(rng.integers(1, 1100))
+        key = (k, n, seed % 3)
+        if key not in cache:
+            if len(cache) > 40:
+                cache.clear()
+            b, s = bench.make_weights(k, n, gpu, gen)
+            cache[key] = (b, s, ops.w4a16_dequant(b, s, n, k).double())
+        b, s, w = cache[key]
+        lda = k + 8 * int(rng.integers(0, 5)) * int(rng.integers(0, 2))
+        x = torch.randn((m, lda), device=gpu, generator=gen).half()[:, :k]
+        ws = workspace_for(n, gpu)
+        mode = int(rng.integers(0, 4))
+        what = f"seed {seed}: m={m} k={k} n={n} lda={lda} mode={mode}"
+        ref = x.double() @ w
+        plain32 = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k, out_f32=True, flags=WIDE)
+        assert float((plain32.double() - ref).abs().max()) < 3e-4, what
+        plain16 = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k, flags=WIDE)
+        assert torch.equal(plain16, plain32.half()), what
+        if mode == 1:
+            n_out = n - 8 * int(rng.integers(0, 20))
+            bias = torch.randn(n_out, device=gpu, generator=gen).half()
+            y = ops.w4a16_linear(x, b, s, ws, n, k, out_features=n_out, bias=bias, flags=WIDE)
+            assert torch.equal(y, plain16[:, :n_out] + bias), what
+        elif mode == 2:
+            res = torch.randn((m, n), device=gpu, generator=gen).half()
+            assert torch.equal(ops.w4a16_linear(x, b, s, ws, n, k, residual=res, flags=WIDE), res + plain16), what
+        elif mode == 3:
+            y = ops.w4a16_linear(x, b, s, ws, n, k, silu_mul=True, out_f32=True, flags=WIDE).double()
+            v = ref.view(m, n // 128, 2, 64)
+            g, u = v[:, :, 0].reshape(m, n // 2), v[:, :, 1].reshape(m, n // 2)
+            want = g / (1 + torch.exp(-g)) * u
+            assert float((y - want).abs().max()) < 1e-3 * max(1.0, float(want.abs().max())), what
