@@ -428,8 +428,8 @@ __global__ __launch_bounds__(256 * KW, 1) void w4a16_tile_kernel(const TileArgs 
         read_xa(xa0, 0, 0);
         bw = expand(0, 0);
     }
-    int slot = 0;
-    for (int it = 0; it < ngroups; ++it) {
+    // one iteration; called with a literal `slot` the ring addresses are constants
+    auto iteration = [&](int it, int slot) __attribute__((always_inline)) {
         const int slot_next = slot + 1 == kRing ? 0 : slot + 1;
         const int slot_prev = slot == 0 ? kRing - 1 : slot - 1;   // holds stage it+2
         half_stage(0, xa0, bw, kDmaA, kDmaB, group_or_last(g_begin + KW * (it + 2)), slot_prev, [&](int i) __attribute__((always_inline)) {
@@ -447,8 +447,15 @@ __global__ __launch_bounds__(256 * KW, 1) void w4a16_tile_kernel(const TileArgs 
             pw[0][t][1] = pw[1][t][1];
         }
         scv[0] = scv[1];
-        slot = slot_next;
+    };
+    // three iterations at a time walk the ring once: every LDS address in them is a constant
+    int it = 0;
+    for (; it + kRing <= ngroups; it += kRing) {
+        iteration(it, 0);
+        iteration(it + 1, 1);
+        iteration(it + 2, 2);
     }
+    for (int slot = 0; it < ngroups; ++it, ++slot) iteration(it, slot);
     UNIQL_WAIT_VMCNT(0);
     __syncthreads();
 
