@@ -84,3 +84,29 @@ def test_static_limit_is_reported(gpu):
     assert lib.uniql_w4a16_gemm_static(None, 4096, fake, fake, fake, None, 0, 1, 4096, 4096, 32, 0, 1.0, 0, None) == -1
     assert lib.uniql_w4a16_gemm_static(None, 4096, None, None, None, None, 0, 0, 4096, 4096, 32, 0, 1.0, 0, None) == 0
     torch.cuda.synchronize()
+
+
+def test_static_entry_point_in_a_graph(gpu):
+    """the callers it is for: a captured graph replays the call (its clearing of the exchange words
+    is a kernel, not a memset) and every replay gives the eager result, with other calls on the
+    array between the replays"""
+    m, k, n = 4, 4096, 4096
+    p = H.make_linear_problem(m, k, n, seed=H.SEED + 7)
+    x, b, s = H.to_gpu(p, gpu)
+    ws = H.workspace_for(n, gpu)
+    want = ops.w4a16_gemm_ex(x, b, s, ws, m, n, k)
+    out = torch.zeros((m, n), dtype=torch.float16, device=gpu)
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        ops.w4a16_gemm_static(x, b, s, ws, out, m, n, k)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        ops.w4a16_gemm_static(x, b, s, ws, out, m, n, k)
+    for i in range(4):
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, want), f"replay {i}"
+        run_pair(gpu, 64, 4096, 1024, flags=(4 << 8) | (1 << 16))   # the tiled kernel's partial tiles in between
