@@ -250,3 +250,125 @@ def test_slice_mamba_in_and_out_proj(gpu):
     assert np.array_equal(cb.cpu().numpy(), want.astype(np.float32)) and cw.shape[0] == len(want)
     nw = slicing.slice_norm(torch.arange(inter, dtype=torch.float32, device=gpu), n_groups, num_heads, inter, load_inter)
     assert np.array_equal(nw.cpu().numpy(), heads.astype(np.float32))
+
+
+def test_slice_quantized_weights_walks_a_model(gpu):
+    """modeling_helpers.py:235-358: the walk over the decoder layers hands every block's tensors to
+    the cut that belongs to them, with the block's own sizes, and leaves everything else alone.
+    Duck-typed stand-ins for the reference's model and helper objects; the cuts themselves are held
+    to the reference's outputs elsewhere."""
+    from types import SimpleNamespace as NS
+    from uniql_amd import slicing
+
+    hidden, inter, heads, kv_heads, head_dim = 256, 512, 4, 2, 64
+    red_inter, red_head = 384, 48
+    m_groups, m_heads, m_inter, m_state, m_red_inter, m_red_state = 2, 8, 512, 64, 384, 48
+
+    def packed(k, n, seed):
+        _, _, p, sp, ws = _full_layer(k, n, seed, gpu)
+        return {"weight": p, "scale": sp, "workspace": ws}
+
+    state, seed = {}, 100
+    def add(key, k, n, bias=False):
+        nonlocal seed
+        seed += 1
+        for name, t in packed(k, n, seed).items():
+            state[f"{key}.{name}"] = t
+        if bias:
+            state[f"{key}.bias"] = torch.arange(n, dtype=torch.float16, device=gpu)
+
+    add("L0.mlp.up_proj", hidden, inter)
+    add("L0.mlp.gate_proj", hidden, inter)
+    add("L0.mlp.down_proj", inter, hidden)
+    add("L0.attn.q_proj", hidden, heads * head_dim, bias=True)
+    add("L0.attn.k_proj", hidden, 256, bias=True)          # 2 x 64 = 128 columns, padded to 256
+    add("L0.attn.v_proj", hidden, 256)
+    add("L0.attn.o_proj", heads * head_dim, hidden)
+    state["L0.attn.indices"] = torch.arange(head_dim, device=gpu).repeat(heads, 1)
+    proj = 2 * m_inter + 2 * m_groups * m_state + m_heads
+    add("L1.mixer.in_proj", hidden, proj + (-proj) % 256)
+    add("L1.mixer.out_proj", m_inter, hidden)
+    conv_ch = m_inter + 2 * m_groups * m_state
+    state["L1.mixer.conv1d.weight"] = torch.arange(conv_ch * 4, dtype=torch.float32, device=gpu).reshape(-1, 1, 4)
+    state["L1.mixer.conv1d.bias"] = torch.arange(conv_ch, dtype=torch.float32, device=gpu)
+    state["L1.mixer.norm.weight"] = torch.arange(m_inter, dtype=torch.float32, device=gpu)
+    state["embed.weight"] = torch.ones(4, device=gpu)
+    before = {k: v.clone() for k, v in state.items()}
+
+    def shape_of(t):
+        return NS(weight=NS(shape=t.shape))
+
+    # what the single cuts return on the untouched tensors (they also give the reduced model's shapes)
+    def cut3(fn, key, *args, **kw):
+        return fn(before[f"{key}.weight"], before[f"{key}.scale"], before[f"{key}.workspace"], *args, **kw)
+    want = {}
+    for proj_name in ("up_proj", "gate_proj"):
+        want[f"L0.mlp.{proj_name}"] = cut3(slicing.slice_w4a16_up_gate_proj, f"L0.mlp.{proj_name}", hidden, inter, red_inter,
+                                            before[f"L0.mlp.{proj_name}.weight"].shape)
+    want["L0.mlp.down_proj"] = cut3(slicing.slice_w4a16_down_proj, "L0.mlp.down_proj", hidden, inter, red_inter,
+                                    before["L0.mlp.down_proj.weight"].shape)
+    qk = {}
+    for proj_name, nh in (("q_proj", heads), ("k_proj", kv_heads)):
+        key = f"L0.attn.{proj_name}"
+        qk[key] = slicing.slice_w4a16_qk_proj(before[f"{key}.weight"], before[f"{key}.bias"], before[f"{key}.scale"],
+                                              before[f"{key}.workspace"], hidden, nh, head_dim, red_head,
+                                              before[f"{key}.weight"].shape)
+    want["L0.attn.v_proj"] = cut3(slicing.slice_w4a16_v_proj, "L0.attn.v_proj", hidden, kv_heads, head_dim, red_head,
+                                  before["L0.attn.v_proj.weight"].shape)
+    want["L0.attn.o_proj"] = cut3(slicing.slice_w4a16_o_proj, "L0.attn.o_proj", hidden, heads, head_dim, red_head,
+                                  before["L0.attn.o_proj.weight"].shape)
+    want["L1.mixer.in_proj"] = cut3(slicing.slice_w4a16_in_proj, "L1.mixer.in_proj", hidden_size=hidden, n_groups=m_groups,
+                                    num_heads=m_heads, intermediate_size=m_inter, ssm_state_size=m_state,
+                                    load_intermediate_size=m_red_inter, load_ssm_state_size=m_red_state,
+                                    load_shape=before["L1.mixer.in_proj.weight"].shape)
+    want["L1.mixer.out_proj"] = cut3(slicing.slice_w4a16_out_proj, "L1.mixer.out_proj", hidden_size=hidden, n_groups=m_groups,
+                                     num_heads=m_heads, intermediate_size=m_inter, load_intermediate_size=m_red_inter,
+                                     load_shape=before["L1.mixer.out_proj.weight"].shape)
+
+    class FakeMlp:
+        intermediate_size = red_inter
+        up_proj = shape_of(before["L0.mlp.up_proj.weight"])
+        gate_proj = shape_of(before["L0.mlp.gate_proj.weight"])
+        down_proj = shape_of(before["L0.mlp.down_proj.weight"])
+
+    class FakeAttn:
+        head_dim = red_head
+        q_proj = shape_of(before["L0.attn.q_proj.weight"])
+        k_proj = shape_of(before["L0.attn.k_proj.weight"])
+        v_proj = shape_of(before["L0.attn.v_proj.weight"])
+        o_proj = shape_of(before["L0.attn.o_proj.weight"])
+
+    class FakeMamba:
+        n_groups, num_heads, intermediate_size, ssm_state_size = m_groups, m_heads, m_red_inter, m_red_state
+        in_proj = shape_of(before["L1.mixer.in_proj.weight"])
+        out_proj = shape_of(before["L1.mixer.out_proj.weight"])
+
+    class Other:
+        pass
+
+    layers = [NS(named_children=lambda: [("mlp", FakeMlp()), ("self_attn", FakeAttn()), ("norm", Other())]),
+              NS(named_children=lambda: [("mixer", FakeMamba())])]
+    model = NS(config=NS(hidden_size=hidden, intermediate_size=inter, num_attention_heads=heads,
+                         num_key_value_heads=kv_heads, head_dim=head_dim), layers=layers)
+    helper = NS(get_layers=lambda m: m.layers, mlp_w4a16_uniql_class_name="FakeMlp",
+                attn_w4a16_uniql_class_name="FakeAttn", mamba_w4a16_uniql_class_name="FakeMamba",
+                get_mlp_key=lambda i: f"L{i}.mlp", get_attn_key=lambda i: f"L{i}.attn", get_mamba_key=lambda i: f"L{i}.mixer",
+                get_mamba_full_intermediate_size=m_inter, get_mamba_full_ssm_state_size=m_state)
+
+    out = slicing.slice_quantized_weights(model, helper, state)
+    assert out is state
+    for key, (w, s, ws) in want.items():
+        assert torch.equal(out[f"{key}.weight"], w) and torch.equal(out[f"{key}.scale"], s), key
+        assert torch.equal(out[f"{key}.workspace"], ws), key
+    for key, (w, b, s, ws) in qk.items():
+        assert torch.equal(out[f"{key}.weight"], w) and torch.equal(out[f"{key}.bias"], b), key
+        assert torch.equal(out[f"{key}.scale"], s) and torch.equal(out[f"{key}.workspace"], ws), key
+    assert torch.equal(out["L0.attn.indices"], slicing.slice_indices(before["L0.attn.indices"], head_dim, red_head))
+    cw, cb = slicing.slice_conv1d(before["L1.mixer.conv1d.weight"], before["L1.mixer.conv1d.bias"], m_groups, m_heads,
+                                  m_inter, m_state, m_red_inter, m_red_state)
+    assert torch.equal(out["L1.mixer.conv1d.weight"], cw) and torch.equal(out["L1.mixer.conv1d.bias"], cb)
+    assert torch.equal(out["L1.mixer.norm.weight"],
+                       slicing.slice_norm(before["L1.mixer.norm.weight"], m_groups, m_heads, m_inter, m_red_inter))
+    assert torch.equal(out["embed.weight"], before["embed.weight"]) and set(out) == set(before)
+    # the cut MLP still computes the kept columns
+    assert out["L0.mlp.up_proj.weight"].shape[1] == 2 * 512 and out["L0.mlp.down_proj.weight"].shape[0] == red_inter // 16

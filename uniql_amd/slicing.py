@@ -226,3 +226,83 @@ def slice_norm(weight, n_groups, num_heads, intermediate_size, load_intermediate
     idx = get_topk_head_indices(n_groups, num_heads, intermediate_size // num_heads,
                                 load_intermediate_size // num_heads, weight.device)
     return weight[idx].contiguous()
+
+
+# ---------------------------------------------------------------------------------------------
+# The walk over a model (modeling_helpers.py:235-358): for every decoder layer, the block that is a
+# UniQL W4A16 MLP / attention / Mamba block gets the tensors of the full-size checkpoint
+# (`loaded_model`, a name -> tensor dict) replaced by their cuts to the block's own sizes.
+# `model` and `model_helper` are the reference's objects, used through the same attributes the
+# reference uses (get_layers, *_w4a16_uniql_class_name, get_*_key, model.config, the blocks' sizes
+# and the shapes of their packed weights); nothing else of them is touched.
+def _replace(state, key, names, values):
+    for name, value in zip(names, values):
+        if value is not None:
+            state[f"{key}.{name}"] = value
+
+
+def _packed(state, key):
+    return state[f"{key}.weight"], state[f"{key}.scale"], state[f"{key}.workspace"]
+
+
+_WSW = ("weight", "scale", "workspace")
+_WBSW = ("weight", "bias", "scale", "workspace")
+
+
+def slice_quantized_weights(model, model_helper, loaded_model):
+    cfg = model.config
+    for layer_idx, layer in enumerate(model_helper.get_layers(model)):
+        for _, block in layer.named_children():
+            kind = block.__class__.__name__
+            if kind == model_helper.mlp_w4a16_uniql_class_name:
+                base = model_helper.get_mlp_key(layer_idx)
+                sizes = (cfg.hidden_size, cfg.intermediate_size, block.intermediate_size)
+                for proj in ("up_proj", "gate_proj"):  # models without a gate have no gate_proj tensors
+                    key = f"{base}.{proj}"
+                    if f"{key}.weight" in loaded_model:
+                        _replace(loaded_model, key, _WSW, slice_w4a16_up_gate_proj(
+                            *_packed(loaded_model, key), *sizes, getattr(block, proj).weight.shape))
+                key = f"{base}.down_proj"
+                _replace(loaded_model, key, _WSW, slice_w4a16_down_proj(
+                    *_packed(loaded_model, key), *sizes, block.down_proj.weight.shape))
+            elif kind == model_helper.attn_w4a16_uniql_class_name:
+                base = model_helper.get_attn_key(layer_idx)
+                head_dim = getattr(cfg, "head_dim", cfg.hidden_size // cfg.num_attention_heads)
+                heads = {"q_proj": cfg.num_attention_heads, "k_proj": cfg.num_key_value_heads,
+                         "v_proj": cfg.num_key_value_heads, "o_proj": cfg.num_attention_heads}
+                for proj in ("q_proj", "k_proj"):
+                    key = f"{base}.{proj}"
+                    w, s, ws = _packed(loaded_model, key)
+                    _replace(loaded_model, key, _WBSW, slice_w4a16_qk_proj(
+                        w, loaded_model.get(f"{key}.bias"), s, ws, cfg.hidden_size, heads[proj], head_dim,
+                        block.head_dim, getattr(block, proj).weight.shape))
+                for proj, cut in (("v_proj", slice_w4a16_v_proj), ("o_proj", slice_w4a16_o_proj)):
+                    key = f"{base}.{proj}"
+                    _replace(loaded_model, key, _WSW, cut(*_packed(loaded_model, key), cfg.hidden_size, heads[proj],
+                                                          head_dim, block.head_dim, getattr(block, proj).weight.shape))
+                if f"{base}.indices" in loaded_model:
+                    loaded_model[f"{base}.indices"] = slice_indices(loaded_model[f"{base}.indices"], head_dim,
+                                                                    block.head_dim)
+            elif kind == model_helper.mamba_w4a16_uniql_class_name:
+                base = model_helper.get_mamba_key(layer_idx)
+                full_inner = model_helper.get_mamba_full_intermediate_size
+                full_state = model_helper.get_mamba_full_ssm_state_size
+                key = f"{base}.in_proj"
+                _replace(loaded_model, key, _WSW, slice_w4a16_in_proj(
+                    *_packed(loaded_model, key), hidden_size=cfg.hidden_size, n_groups=block.n_groups,
+                    num_heads=block.num_heads, intermediate_size=full_inner, ssm_state_size=full_state,
+                    load_intermediate_size=block.intermediate_size, load_ssm_state_size=block.ssm_state_size,
+                    load_shape=block.in_proj.weight.shape))
+                key = f"{base}.conv1d"
+                _replace(loaded_model, key, ("weight", "bias"), slice_conv1d(
+                    loaded_model[f"{key}.weight"], loaded_model[f"{key}.bias"], block.n_groups, block.num_heads,
+                    full_inner, full_state, block.intermediate_size, block.ssm_state_size))
+                loaded_model[f"{base}.norm.weight"] = slice_norm(
+                    loaded_model[f"{base}.norm.weight"], block.n_groups, block.num_heads, full_inner,
+                    block.intermediate_size)
+                key = f"{base}.out_proj"
+                _replace(loaded_model, key, _WSW, slice_w4a16_out_proj(
+                    *_packed(loaded_model, key), hidden_size=cfg.hidden_size, n_groups=block.n_groups,
+                    num_heads=block.num_heads, intermediate_size=full_inner,
+                    load_intermediate_size=block.intermediate_size, load_shape=block.out_proj.weight.shape))
+    return loaded_model
