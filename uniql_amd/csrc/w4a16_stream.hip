@@ -70,7 +70,7 @@ struct StreamArgs {
 // quad are real, and XQ, how many quads of activation rows are loaded and staged.  WAVES:
 // wavefronts per workgroup (4 or 8); with 8 a workgroup can cover all of K for shapes with
 // many strips, which removes the exchange of partial sums between workgroups.  EXT: the call
-// uses something beyond the plain product (input shorter than K, output cut or strided, bias,
+// uses something beyond the plain product (input shorter than K, output cut, strided or fp32, bias,
 // gated pairs); the plain instantiation leaves all of that code out, which at a few
 // microseconds per launch is measurable (instruction fetch).
 // HAD: 0 no rotation; 1 every 128-block of the activations is rotated in registers while it is
@@ -79,7 +79,7 @@ struct StreamArgs {
 // weights are on their way, and the staging reads its 128 values from there.  Same butterfly
 // order and the same single rounding as the transform kernel: the same values bit for bit.
 template <int RC, int HAD, int WAVES, bool EXT>
-__global__ __launch_bounds__(64 * WAVES, RC == 16 ? 2 : 3)
+__global__ __launch_bounds__(64 * WAVES, 2)
 void w4a16_stream_kernel(const StreamArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     constexpr int NV = RC < 4 ? RC : 4;
@@ -274,24 +274,7 @@ void w4a16_stream_kernel(const StreamArgs a) {
     }
     if (HAD == 2)  // all waves, also those without groups: the transform has workgroup barriers
         fwht_rows_to_lds<kRowChunks>(xin, reinterpret_cast<float*>(lds + a.fwht_lds), a.M, a.K, a.log2K, tid, 64 * WAVES);
-    if (g_begin < g_end) {
-        int g = g_begin;
-        while (g + 2 < g_end) {
-            issue_loads(g + 1, set_b);
-            process(set_a, g);
-            issue_loads(g + 2, set_a);
-            process(set_b, g + 1);
-            g += 2;
-        }
-        if (g + 1 < g_end) {
-            issue_loads(g + 1, set_b);
-            process(set_a, g);
-            process(set_b, g + 1);
-        } else {
-            process(set_a, g);
-        }
-    }
-
+    auto finish = [&]() __attribute__((always_inline)) {
     // ---- combine the waves (fixed order), then the K splits ------------------------------
     // acc[jb][v] on lane l is row m = 4 (l/16) + v, column
     // 128 strip + 64 (slot/8) + 16 (jb/2) + 8 (jb%2) + slot%8.
@@ -299,10 +282,11 @@ void w4a16_stream_kernel(const StreamArgs a) {
     // round.
     float* red = reinterpret_cast<float*>(lds + (size_t)WAVES * a.xrows * kXsStride);
     // the exchange area holds 64 rows of 128 floats: all waves at once up to 8 activation rows
-    const int rr_rows = a.xrows <= 4 ? 4 : (a.xrows <= 8 ? 8 : 16);  // rows per wave in the exchange area
-    const int wpr = 64 / rr_rows < WAVES ? 64 / rr_rows : WAVES;     // waves per round
+    // (the row class fixes both: the staged rows are M rounded up to a multiple of four)
+    constexpr int rr_rows = RC <= 4 ? 4 : RC;                            // rows per wave in the exchange area
+    constexpr int wpr = 64 / rr_rows < WAVES ? 64 / rr_rows : WAVES;     // waves per round
     constexpr int RPT = WAVES / 2;                  // output rows covered per pass of the workgroup
-    constexpr int NI = 16 / RPT;                    // passes needed for 16 rows
+    constexpr int NI = (RC + RPT - 1) / RPT;        // passes needed for the rows of this row class
     const int ncol_lane = 64 * (slot >> 3) + c8;
     const int col_out = tid & 127;
     const int n_out = 128 * strip + col_out;
@@ -315,15 +299,15 @@ void w4a16_stream_kernel(const StreamArgs a) {
     for (int round = 0; round < WAVES / wpr; ++round) {
         if (!first_round) __syncthreads();
         first_round = false;
-        if (w / wpr == round) {
+        // (one condition around all of a lane's writes: rows from M up to the area's rr_rows per wave
+        // are written too and never read; a condition per write would put every write behind a branch)
+        if (w / wpr == round && 4 * kq < rr_rows) {
 #pragma unroll
             for (int jb = 0; jb < 8; ++jb) {
 #pragma unroll
                 for (int v = 0; v < NV; ++v) {
                     const int ml = 4 * kq + v;
-                    if (ml < a.M)
-                        red[((w % wpr) * rr_rows + ml) * 128 + ncol_lane + 16 * (jb >> 1) + 8 * (jb & 1)] =
-                            acc[jb][v];
+                    red[((w % wpr) * rr_rows + ml) * 128 + ncol_lane + 16 * (jb >> 1) + 8 * (jb & 1)] = acc[jb][v];
                 }
             }
         }
@@ -333,11 +317,9 @@ void w4a16_stream_kernel(const StreamArgs a) {
             const int ml = (tid >> 7) + RPT * i;
             if (ml < a.M) {
 #pragma unroll
-                for (int ww = 0; ww < WAVES; ++ww) {
-                    if (ww < wpr) {
-                        tot[i] += red[(ww * rr_rows + ml) * 128 + col_out];
-                        if (gated) oth[i] += red[(ww * rr_rows + ml) * 128 + col_pair];
-                    }
+                for (int ww = 0; ww < wpr; ++ww) {
+                    tot[i] += red[(ww * rr_rows + ml) * 128 + col_out];
+                    if (gated) oth[i] += red[(ww * rr_rows + ml) * 128 + col_pair];
                 }
             }
         }
@@ -353,9 +335,7 @@ void w4a16_stream_kernel(const StreamArgs a) {
             if (mine) {
                 if constexpr (EXT) {
                     finish_store(a.epi, a.D, m, n_out, total);
-                } else if (a.epi.out_f32) {
-                    reinterpret_cast<float*>(a.D)[(size_t)m * a.N + n_out] = total;
-                } else {
+                } else {  // (fp32 output is one of the extended instantiation's cases)
                     reinterpret_cast<half_t*>(a.D)[(size_t)m * a.N + n_out] = (half_t)total;
                 }
                 if (a.splits != 1) accum_reset(word);
@@ -372,6 +352,36 @@ void w4a16_stream_kernel(const StreamArgs a) {
                 }
             }
         }
+    }
+    };
+
+    // The short cases come first in the code: a wave with one or two groups runs through the kernel
+    // once, on instructions that arrive from memory as it goes, and should meet them in fetch order.
+    if (g_begin + 1 >= g_end) {
+        if (g_begin < g_end) process(set_a, g_begin);
+        finish();
+    } else if (g_begin + 2 >= g_end) {
+        issue_loads(g_begin + 1, set_b);
+        process(set_a, g_begin);
+        process(set_b, g_begin + 1);
+        finish();
+    } else {
+        int g = g_begin;
+        while (g + 2 < g_end) {
+            issue_loads(g + 1, set_b);
+            process(set_a, g);
+            issue_loads(g + 2, set_a);
+            process(set_b, g + 1);
+            g += 2;
+        }
+        if (g + 1 < g_end) {
+            issue_loads(g + 1, set_b);
+            process(set_a, g);
+            process(set_b, g + 1);
+        } else {
+            process(set_a, g);
+        }
+        finish();
     }
 }
 
@@ -437,8 +447,8 @@ size_t stream_accum_bytes(int m, int n, int k) {
 template <int RC, int HAD, int WAVES, bool EXT>
 static hipError_t launch_one(StreamArgs a, hipStream_t stream) {
     const size_t stage = (size_t)WAVES * a.xrows * kXsStride * 4;
-    const int rr_rows = a.xrows <= 4 ? 4 : (a.xrows <= 8 ? 8 : 16);
-    const int wpr = 64 / rr_rows < WAVES ? 64 / rr_rows : WAVES;
+    constexpr int rr_rows = RC <= 4 ? 4 : RC;  // as in the kernel
+    constexpr int wpr = 64 / rr_rows < WAVES ? 64 / rr_rows : WAVES;
     const size_t red = (size_t)wpr * rr_rows * 128 * 4;
     size_t shmem = stage + red;
     if (HAD == 2) {  // one padded fp32 image per activation row behind the staging and exchange areas
@@ -472,7 +482,7 @@ template <int HAD>
 static hipError_t launch_rows(const StreamArgs& a, int waves, hipStream_t stream) {
     const Epilogue& e = a.epi;
     const bool ext = e.gated || e.bias || e.residual || e.relu2 || e.transpose || e.n_store != a.N ||
-                     e.ldd != a.N || a.k_valid != a.K;
+                     e.ldd != a.N || a.k_valid != a.K || e.out_f32;
     if (a.M == 1) return launch_waves<1, HAD>(a, waves, ext, stream);
     if (a.M == 2) return launch_waves<2, HAD>(a, waves, ext, stream);
     if (a.M <= 4) return launch_waves<4, HAD>(a, waves, ext, stream);
