@@ -403,7 +403,8 @@ struct StreamPlan {
 //     allows it (long streams per wave, two register sets in flight), else eight waves;
 //   * otherwise K is split over workgroups.  One or two rows: 4 waves, and as many groups per wave
 //     as it takes to stay within about 288 workgroups.  More rows: every split costs a 64-bit
-//     atomic per output element, so 8 waves (4 for small problems) and at most 256 workgroups.
+//     atomic per output element, so 8 waves (4 for small problems: below 1536 units, from 8 rows on
+//     below 768) and at most 256 workgroups.
 static StreamPlan stream_plan(int m, int n, int k, int upw_override, int waves_override) {
     const int nstrips = n / 128, G = k / 128;
     const int64_t units = (int64_t)nstrips * G;
@@ -417,7 +418,7 @@ static StreamPlan stream_plan(int m, int n, int k, int upw_override, int waves_o
     } else if (m <= 2) {
         p.waves = 4;
     } else {
-        p.waves = (m <= 16 && units >= 1536) ? 8 : 4;
+        p.waves = (m <= 16 && units >= (m >= 8 ? 768 : 1536)) ? 8 : 4;
         max_wgs = 256;
     }
     if (upw_override > 0) {
@@ -427,6 +428,10 @@ static StreamPlan stream_plan(int m, int n, int k, int upw_override, int waves_o
     } else {
         p.upw = 1;
         while (p.upw < 8 && (int64_t)nstrips * ceil_div(G, p.waves * p.upw) > max_wgs) ++p.upw;
+        // one or two rows and a strip count that lands well below the chip's 256 compute units once
+        // the grid is inside the limit (146 strips: 292 workgroups are too many, 146 too few): one
+        // group per wave and many short workgroups instead (4096 -> 18688 at one row: 10.5 against 11.3 us)
+        if (m <= 2 && p.upw > 1 && (int64_t)nstrips * ceil_div(G, p.waves * p.upw) < 176) p.upw = 1;
     }
     p.splits = ceil_div(G, p.waves * p.upw);
     while (p.splits > kAccumMaxSplits) {  // the contribution count has 7 bits
