@@ -153,6 +153,112 @@ __device__ __forceinline__ void finish_store_gated(const Epilogue& e, void* D, i
     }
 }
 
+// Eight consecutive fp16 values from p: one 16-byte load where the address allows it.
+__device__ __forceinline__ void load_eight(const half_t* p, bool aligned16, float (&out)[8]) {
+    if (aligned16) {
+        const h8 v = *reinterpret_cast<const h8*>(p);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] = (float)v[i];
+    } else {
+#pragma unroll
+        for (int i = 0; i < 8; ++i) out[i] = (float)p[i];
+    }
+}
+
+// Eight consecutive outputs of row m starting at column n0 (a multiple of 8): one 16-byte
+// store where the output's layout allows it, element stores otherwise.  Bias and residual come as
+// 16-byte loads where they are aligned; the roundings are those of finish_half / finish_half_gated.
+__device__ __forceinline__ void store_eight(const Epilogue& e, void* D, int m, int n0, f4 lo, f4 hi) {
+    if (e.vec_ok && n0 + 8 <= e.n_store) {
+        const size_t o = (size_t)m * e.ldd + n0;
+        if (e.out_f32 && !e.bias && !e.residual && !e.relu2) {
+            float* d = reinterpret_cast<float*>(D) + o;
+            *reinterpret_cast<f4*>(d) = lo;
+            *reinterpret_cast<f4*>(d + 4) = hi;
+            return;
+        }
+        if (!e.out_f32 && !e.bias && !e.residual && !e.relu2) {
+            const h2 r0 = h2{(half_t)lo[0], (half_t)lo[1]}, r1 = h2{(half_t)lo[2], (half_t)lo[3]};
+            const h2 r2 = h2{(half_t)hi[0], (half_t)hi[1]}, r3 = h2{(half_t)hi[2], (half_t)hi[3]};
+            *reinterpret_cast<u32x4*>(reinterpret_cast<half_t*>(D) + o) =
+                u32x4{h2_to_bits(r0), h2_to_bits(r1), h2_to_bits(r2), h2_to_bits(r3)};
+            return;
+        }
+        if (!e.out_f32) {
+            half_t r[8];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                r[i] = (half_t)lo[i];
+                r[4 + i] = (half_t)hi[i];
+            }
+            if (e.bias) {
+                float b[8];
+                load_eight(e.bias + n0, (reinterpret_cast<uintptr_t>(e.bias) & 15u) == 0, b);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) r[i] = (half_t)((float)r[i] + b[i]);
+            }
+            if (e.relu2) {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const float p = (float)r[i] > 0.f ? (float)r[i] : 0.f;
+                    r[i] = (half_t)(p * p);
+                }
+            }
+            if (e.residual) {
+                float q[8];
+                load_eight(e.residual + (size_t)m * e.ldr + n0,
+                           (reinterpret_cast<uintptr_t>(e.residual) & 15u) == 0 && (e.ldr & 7) == 0, q);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) r[i] = (half_t)(q[i] + (float)r[i]);
+            }
+            *reinterpret_cast<h8*>(reinterpret_cast<half_t*>(D) + o) = h8{r[0], r[1], r[2], r[3], r[4], r[5], r[6], r[7]};
+            return;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        finish_store(e, D, m, n0 + i, lo[i]);
+        finish_store(e, D, m, n0 + 4 + i, hi[i]);
+    }
+}
+__device__ __forceinline__ void store_eight_gated(const Epilogue& e, void* D, int m, int n0, f4 glo, f4 ghi, f4 ulo,
+                                                  f4 uhi) {
+    if (e.vec_ok && !e.out_f32 && n0 + 8 <= e.n_store) {
+        half_t r[8], g16[8], u16[8];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            g16[i] = (half_t)glo[i];
+            g16[4 + i] = (half_t)ghi[i];
+            u16[i] = (half_t)ulo[i];
+            u16[4 + i] = (half_t)uhi[i];
+        }
+        if (e.bias) {
+            float bg[8], bu[8];
+            const bool al = (reinterpret_cast<uintptr_t>(e.bias) & 15u) == 0;
+            load_eight(e.bias + n0, al, bg);
+            load_eight(e.bias + e.n_store + n0, al && (e.n_store & 7) == 0, bu);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                g16[i] = (half_t)((float)g16[i] + bg[i]);
+                u16[i] = (half_t)((float)u16[i] + bu[i]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const half_t a16 = (half_t)silu_f32((float)g16[i]);
+            r[i] = (half_t)((float)a16 * (float)u16[i]);
+        }
+        *reinterpret_cast<h8*>(reinterpret_cast<half_t*>(D) + (size_t)m * e.ldd + n0) =
+            h8{r[0], r[1], r[2], r[3], r[4], r[5], r[6], r[7]};
+        return;
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        finish_store_gated(e, D, m, n0 + i, glo[i], ulo[i]);
+        finish_store_gated(e, D, m, n0 + 4 + i, ghi[i], uhi[i]);
+    }
+}
+
 // ---- exchange of partial sums between workgroups that split K ------------------------
 // One 64-bit word per output element in a zero-initialised buffer:
 //   bits 14..63  the running sum in units of 2^-24 (two's complement, 50 bits),

@@ -72,61 +72,6 @@ __device__ __forceinline__ void buffer_to_lds16(__amdgpu_buffer_rsrc_t rsrc, uin
 // s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding)
 #define UNIQL_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
 
-// Eight consecutive outputs of row m starting at column n0 (a multiple of 8): one 16-byte
-// store where the output's layout allows it, element stores otherwise.
-__device__ __forceinline__ void store_eight(const Epilogue& e, void* D, int m, int n0, f4 lo, f4 hi) {
-    if (e.vec_ok && n0 + 8 <= e.n_store) {
-        const size_t o = (size_t)m * e.ldd + n0;
-        if (e.out_f32 && !e.bias && !e.residual && !e.relu2) {
-            float* d = reinterpret_cast<float*>(D) + o;
-            *reinterpret_cast<f4*>(d) = lo;
-            *reinterpret_cast<f4*>(d + 4) = hi;
-            return;
-        }
-        if (!e.out_f32 && !e.bias && !e.residual && !e.relu2) {
-            const h2 r0 = h2{(half_t)lo[0], (half_t)lo[1]}, r1 = h2{(half_t)lo[2], (half_t)lo[3]};
-            const h2 r2 = h2{(half_t)hi[0], (half_t)hi[1]}, r3 = h2{(half_t)hi[2], (half_t)hi[3]};
-            *reinterpret_cast<u32x4*>(reinterpret_cast<half_t*>(D) + o) =
-                u32x4{h2_to_bits(r0), h2_to_bits(r1), h2_to_bits(r2), h2_to_bits(r3)};
-            return;
-        }
-        if (!e.out_f32) {
-            half_t r[8];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                r[i] = finish_half(e, m, n0 + i, lo[i]);
-                r[4 + i] = finish_half(e, m, n0 + 4 + i, hi[i]);
-            }
-            *reinterpret_cast<h8*>(reinterpret_cast<half_t*>(D) + o) = h8{r[0], r[1], r[2], r[3], r[4], r[5], r[6], r[7]};
-            return;
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        finish_store(e, D, m, n0 + i, lo[i]);
-        finish_store(e, D, m, n0 + 4 + i, hi[i]);
-    }
-}
-__device__ __forceinline__ void store_eight_gated(const Epilogue& e, void* D, int m, int n0, f4 glo, f4 ghi, f4 ulo,
-                                                  f4 uhi) {
-    if (e.vec_ok && !e.out_f32 && n0 + 8 <= e.n_store) {
-        half_t r[8];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            r[i] = finish_half_gated(e, n0 + i, glo[i], ulo[i]);
-            r[4 + i] = finish_half_gated(e, n0 + 4 + i, ghi[i], uhi[i]);
-        }
-        *reinterpret_cast<h8*>(reinterpret_cast<half_t*>(D) + (size_t)m * e.ldd + n0) =
-            h8{r[0], r[1], r[2], r[3], r[4], r[5], r[6], r[7]};
-        return;
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        finish_store_gated(e, D, m, n0 + i, glo[i], ulo[i]);
-        finish_store_gated(e, D, m, n0 + 4 + i, ghi[i], uhi[i]);
-    }
-}
-
 // Eight fp32 partial sums to / from a workgroup's slot of the split-K scratch area: relaxed
 // device-scope accesses (write-through stores, loads that do not trust a stale cache line), so
 // workgroups on different XCDs exchange them without flushing or invalidating a whole L2.  The

@@ -82,95 +82,6 @@ __device__ __forceinline__ int wide_sw(int x) { return (((x >> 2) ^ (x >> 4)) & 
 // X rows are 128 bytes (eight 16-byte chunks): chunk c of row x sits at position c ^ sw8(x)
 __device__ __forceinline__ int wide_sw8(int x) { return (x >> 1) & 7; }
 
-// Four consecutive fp16 values from p: one 8-byte load where the address allows it.
-__device__ __forceinline__ void wide_load_four(const half_t* p, bool aligned8, float (&out)[4]) {
-    if (aligned8) {
-        const wide_u32x2 w = *reinterpret_cast<const wide_u32x2*>(p);
-        const h2 a = bits_to_h2(w.x), b = bits_to_h2(w.y);
-        out[0] = (float)a.x;
-        out[1] = (float)a.y;
-        out[2] = (float)b.x;
-        out[3] = (float)b.y;
-    } else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) out[i] = (float)p[i];
-    }
-}
-
-// Four consecutive outputs of row m starting at column n0 (a multiple of 4): one 8- or 16-byte
-// store where the output's layout allows it, element stores otherwise.  The roundings are those of
-// finish_half / finish_half_gated; bias and residual come as 8-byte loads where they are aligned.
-__device__ __forceinline__ void wide_store_four(const Epilogue& e, void* D, int m, int n0, f4 v) {
-    if (e.vec_ok && n0 + 4 <= e.n_store) {
-        const size_t o = (size_t)m * e.ldd + n0;
-        if (e.out_f32 && !e.bias && !e.residual && !e.relu2) {
-            *reinterpret_cast<f4*>(reinterpret_cast<float*>(D) + o) = v;
-            return;
-        }
-        if (!e.out_f32) {
-            half_t y[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) y[i] = (half_t)v[i];
-            if (e.bias) {
-                float b[4];
-                wide_load_four(e.bias + n0, (reinterpret_cast<uintptr_t>(e.bias) & 7u) == 0, b);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) y[i] = (half_t)((float)y[i] + b[i]);
-            }
-            if (e.relu2) {
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float r = (float)y[i] > 0.f ? (float)y[i] : 0.f;
-                    y[i] = (half_t)(r * r);
-                }
-            }
-            if (e.residual) {
-                float r[4];
-                wide_load_four(e.residual + (size_t)m * e.ldr + n0,
-                               (reinterpret_cast<uintptr_t>(e.residual) & 7u) == 0 && (e.ldr & 3) == 0, r);
-#pragma unroll
-                for (int i = 0; i < 4; ++i) y[i] = (half_t)(r[i] + (float)y[i]);
-            }
-            *reinterpret_cast<wide_u32x2*>(reinterpret_cast<half_t*>(D) + o) =
-                wide_u32x2{h2_to_bits(h2{y[0], y[1]}), h2_to_bits(h2{y[2], y[3]})};
-            return;
-        }
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) finish_store(e, D, m, n0 + i, v[i]);
-}
-__device__ __forceinline__ void wide_store_four_gated(const Epilogue& e, void* D, int m, int n0, f4 g, f4 u) {
-    if (e.vec_ok && !e.out_f32 && n0 + 4 <= e.n_store) {
-        half_t g16[4], u16[4], y[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            g16[i] = (half_t)g[i];
-            u16[i] = (half_t)u[i];
-        }
-        if (e.bias) {
-            float bg[4], bu[4];
-            const bool al = (reinterpret_cast<uintptr_t>(e.bias) & 7u) == 0;
-            wide_load_four(e.bias + n0, al, bg);
-            wide_load_four(e.bias + e.n_store + n0, al && (e.n_store & 3) == 0, bu);
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                g16[i] = (half_t)((float)g16[i] + bg[i]);
-                u16[i] = (half_t)((float)u16[i] + bu[i]);
-            }
-        }
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const half_t a16 = (half_t)silu_f32((float)g16[i]);
-            y[i] = (half_t)((float)a16 * (float)u16[i]);
-        }
-        *reinterpret_cast<wide_u32x2*>(reinterpret_cast<half_t*>(D) + (size_t)m * e.ldd + n0) =
-            wide_u32x2{h2_to_bits(h2{y[0], y[1]}), h2_to_bits(h2{y[2], y[3]})};
-        return;
-    }
-#pragma unroll
-    for (int i = 0; i < 4; ++i) finish_store_gated(e, D, m, n0 + i, g[i], u[i]);
-}
-
 template <int V>
 struct WideInt {
     static constexpr int value = V;
@@ -492,39 +403,79 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
         f(WideInt<2>{});
         f(WideInt<3>{});
     };
-    const bool gated = EXT && a.epi.gated != 0;  // uniform: columns c and c + 64 of the wave's strip are a (gate, up) pair
-    four_times([&](auto mtc) __attribute__((always_inline)) {
-        constexpr int mt = decltype(mtc)::value;
-        const int m = m0 + 128 * wm + 32 * mt + rs;
-        if (m >= a.M) return;
-        four_times([&](auto ntc) __attribute__((always_inline)) {
-            constexpr int nt = decltype(ntc)::value;
-            four_times([&](auto qc) __attribute__((always_inline)) {
-                constexpr int q = decltype(qc)::value;
-                const f16& t = acc[mt][nt];
-                const f4 v = f4{t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
-                if (gated) {
-                    if constexpr (nt < 2) {
-                        const f16& up = acc[mt][nt + 2];
-                        wide_store_four_gated(a.epi, a.D, m, (n0 + 128 * wn) / 2 + 32 * nt + 8 * q + 4 * hs, v,
-                                              f4{up[4 * q], up[4 * q + 1], up[4 * q + 2], up[4 * q + 3]});
+    if constexpr (EXT) {
+        // Everything beyond the plain product: the wave's quarter goes through LDS, 32 rows at a time,
+        // and leaves it as (row, 8 consecutive columns) units through the same store code as the
+        // 128-column kernel, in a loop.  (Straight from the registers the epilogue's cases would
+        // be instantiated once per accumulator quad, 64 times: several hundred KB of code that every
+        // compute unit fetches once per launch, 8 to 34 % of a launch at 1024 to 4096 rows.)
+        __builtin_amdgcn_s_barrier();  // every wave has read its last operands: their LDS is free
+        constexpr int kStride = 132;   // floats per staged row
+        float* const stage = reinterpret_cast<float*>(ldsb) + (size_t)w * 32 * kStride;  // this wave's 32 x 128 block
+        const bool gated = a.epi.gated != 0;  // uniform: columns c and c + 64 of the wave's strip are a (gate, up) pair
+        four_times([&](auto mtc) __attribute__((always_inline)) {
+            constexpr int mt = decltype(mtc)::value;
+            four_times([&](auto ntc) __attribute__((always_inline)) {
+                constexpr int nt = decltype(ntc)::value;
+                four_times([&](auto qc) __attribute__((always_inline)) {
+                    constexpr int q = decltype(qc)::value;
+                    const f16& t = acc[mt][nt];
+                    *reinterpret_cast<f4*>(stage + rs * kStride + 32 * nt + 8 * q + 4 * hs) =
+                        f4{t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
+                });
+            });
+            // LDS operations of one wave complete in issue order: the reads below see the writes above
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            const int mrow = m0 + 128 * wm + 32 * mt;
+            if (!gated) {
+#pragma clang loop unroll(disable)
+                for (int u = 0; u < 8; ++u) {
+                    const int unit = 64 * u + lane_s, row = unit >> 4, c0 = (unit & 15) * 8;
+                    const float* src = stage + row * kStride + c0;
+                    const f4 lo = *reinterpret_cast<const f4*>(src), hi = *reinterpret_cast<const f4*>(src + 4);
+                    if (mrow + row < a.M) store_eight(a.epi, a.D, mrow + row, n0 + 128 * wn + c0, lo, hi);
+                }
+            } else {
+#pragma clang loop unroll(disable)
+                for (int u = 0; u < 4; ++u) {
+                    const int unit = 64 * u + lane_s, row = unit >> 3, c0 = (unit & 7) * 8;
+                    const float* src = stage + row * kStride + c0;
+                    const f4 glo = *reinterpret_cast<const f4*>(src), ghi = *reinterpret_cast<const f4*>(src + 4);
+                    const f4 ulo = *reinterpret_cast<const f4*>(src + 64), uhi = *reinterpret_cast<const f4*>(src + 68);
+                    if (mrow + row < a.M) store_eight_gated(a.epi, a.D, mrow + row, (n0 + 128 * wn) / 2 + c0, glo, ghi, ulo, uhi);
+                }
+            }
+            // the next 32 rows overwrite the block: not before these reads
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        });
+    } else {
+        four_times([&](auto mtc) __attribute__((always_inline)) {
+            constexpr int mt = decltype(mtc)::value;
+            const int m = m0 + 128 * wm + 32 * mt + rs;
+            if (m >= a.M) return;
+            four_times([&](auto ntc) __attribute__((always_inline)) {
+                constexpr int nt = decltype(ntc)::value;
+                four_times([&](auto qc) __attribute__((always_inline)) {
+                    constexpr int q = decltype(qc)::value;
+                    const f16& t = acc[mt][nt];
+                    const f4 v = f4{t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
+                    const int n = n0 + 128 * wn + 32 * nt + 8 * q + 4 * hs;
+                    if (a.epi.out_f32) {
+                        *reinterpret_cast<f4*>(reinterpret_cast<float*>(a.D) + (size_t)m * a.N + n) = v;
+                    } else {
+                        const h2 p0 = h2{(half_t)v[0], (half_t)v[1]};
+                        const h2 p1 = h2{(half_t)v[2], (half_t)v[3]};
+                        *reinterpret_cast<wide_u32x2*>(reinterpret_cast<half_t*>(a.D) + (size_t)m * a.N + n) =
+                            wide_u32x2{h2_to_bits(p0), h2_to_bits(p1)};
                     }
-                    return;
-                }
-                const int n = n0 + 128 * wn + 32 * nt + 8 * q + 4 * hs;
-                if constexpr (EXT) {
-                    wide_store_four(a.epi, a.D, m, n, v);
-                } else if (a.epi.out_f32) {
-                    *reinterpret_cast<f4*>(reinterpret_cast<float*>(a.D) + (size_t)m * a.N + n) = v;
-                } else {
-                    const h2 p0 = h2{(half_t)v[0], (half_t)v[1]};
-                    const h2 p1 = h2{(half_t)v[2], (half_t)v[3]};
-                    *reinterpret_cast<wide_u32x2*>(reinterpret_cast<half_t*>(a.D) + (size_t)m * a.N + n) =
-                        wide_u32x2{h2_to_bits(p0), h2_to_bits(p1)};
-                }
+                });
             });
         });
-    });
+    }
 }
 
 // ---------------------------------------------------------------------------------
