@@ -438,6 +438,10 @@ def main():
                              "hbm_frac": round(linear_bytes(m, layer.k, layer.n) / sec_k / 1e9 / HBM_PEAK_GBS, 4)}
     result["config"]["per_linear"] = floor
     result["config"]["read_floor_us_per_step"] = round(sum(v["read_floor_us"] for v in floor.values()), 2)
+    # what one node of a replayed graph costs when its kernel does nothing (one workgroup fills 64 floats)
+    tiny = torch.zeros(64, device=dev)
+    sec_e, _ = time_graphs(lambda i: tiny.fill_(1.0), 1, 400, 40)
+    result["config"]["empty_kernel_us_per_graph_node"] = round(sec_e * 1e6, 2)
     del layers
     torch.cuda.empty_cache()
 
