@@ -119,9 +119,10 @@ def test_pruned_llama_shapes(gpu, name, in_f, out_f, had, m):
 
 
 # ------------------------------------------------------------------ Mamba2-8B block
-@pytest.mark.parametrize("m", [1, 1024])
+@pytest.mark.parametrize("m", [1, 2, 3, 16, 1024])
 def test_mamba_in_proj(gpu, m):
-    """4096 -> 18560 = 2 * 8192 + 2 * 8 * 128 + 128, padded to 18688 output columns (146 strips)."""
+    """4096 -> 18560 = 2 * 8192 + 2 * 8 * 128 + 128, padded to 18688 output columns (146 strips: at one and
+    two rows the streaming kernel's plan of many one-group workgroups, from three rows on 8 waves)."""
     layer, g = pruned_module(4096, 18560, gpu, seed=4000 + m)
     assert layer.size_n == 18688 and tuple(layer.weight.shape) == (256, 37376)
     x = torch.randn(m, 4096, generator=g, device=gpu).half()
