@@ -43,7 +43,7 @@ LLC_BYTES = 256 << 20
 # HBM bytes per launch of the default workload (mean over the four linears) from two
 # rocprofv3 --pmc runs of this file, FETCH_SIZE and WRITE_SIZE, each scaled by the reading for a
 # 128 MiB elementwise copy (--pmc-calibrate): factors 2.000 and 1.000.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28685125
+MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28685090
 
 LLAMA_DECODE = [("qkv", 4096, 6144), ("o_proj", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
 PRUNED = [("q_pruned", 4096, 3584, 0), ("o_pruned", 3456, 4096, 0), ("gate_up_pruned", 4096, 24320, 0),

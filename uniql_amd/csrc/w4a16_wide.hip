@@ -58,7 +58,6 @@ struct WideArgs {
 };
 
 typedef __attribute__((address_space(3))) void* wide_lptr_t;
-typedef uint32_t wide_u32x2 __attribute__((ext_vector_type(2)));
 
 // s_waitcnt vmcnt(n) with the other counters left alone (gfx9 encoding)
 #define UNIQL_WIDE_WAIT_VMCNT(n) __builtin_amdgcn_s_waitcnt(((n) & 15) | (((n) >> 4) << 14) | 0x0F70)
@@ -87,7 +86,6 @@ struct WideInt {
     static constexpr int value = V;
 };
 
-template <bool EXT>
 __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint32_t lds[];
     char* const ldsb = reinterpret_cast<char*>(lds);
@@ -403,79 +401,56 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
         f(WideInt<2>{});
         f(WideInt<3>{});
     };
-    if constexpr (EXT) {
-        // Everything beyond the plain product: the wave's quarter goes through LDS, 32 rows at a time,
-        // and leaves it as (row, 8 consecutive columns) units through the same store code as the
-        // 128-column kernel, in a loop.  (Straight from the registers the epilogue's cases would
-        // be instantiated once per accumulator quad, 64 times: several hundred KB of code that every
-        // compute unit fetches once per launch, 8 to 34 % of a launch at 1024 to 4096 rows.)
-        __builtin_amdgcn_s_barrier();  // every wave has read its last operands: their LDS is free
-        constexpr int kStride = 132;   // floats per staged row
-        float* const stage = reinterpret_cast<float*>(ldsb) + (size_t)w * 32 * kStride;  // this wave's 32 x 128 block
-        const bool gated = a.epi.gated != 0;  // uniform: columns c and c + 64 of the wave's strip are a (gate, up) pair
-        four_times([&](auto mtc) __attribute__((always_inline)) {
-            constexpr int mt = decltype(mtc)::value;
-            four_times([&](auto ntc) __attribute__((always_inline)) {
-                constexpr int nt = decltype(ntc)::value;
-                four_times([&](auto qc) __attribute__((always_inline)) {
-                    constexpr int q = decltype(qc)::value;
-                    const f16& t = acc[mt][nt];
-                    *reinterpret_cast<f4*>(stage + rs * kStride + 32 * nt + 8 * q + 4 * hs) =
-                        f4{t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
-                });
+    // The wave's quarter goes through LDS, 32 rows at a time, and leaves it as (row, 8 consecutive
+    // columns) units through the same store code as the 128-column kernel, in a loop: 16 lanes write
+    // 256 contiguous bytes of an output row.  (Straight from the registers a store instruction
+    // writes 16 bytes to each of 32 rows, 1-2.5 % of a launch slower even for the plain product, and
+    // the epilogue's cases would be instantiated once per accumulator quad, 64 times: several
+    // hundred KB of code that every compute unit fetches once per launch, 8 to 34 % of a launch
+    // at 1024 to 4096 rows.)
+    __builtin_amdgcn_s_barrier();  // every wave has read its last operands: their LDS is free
+    constexpr int kStride = 132;   // floats per staged row
+    float* const stage = reinterpret_cast<float*>(ldsb) + (size_t)w * 32 * kStride;  // this wave's 32 x 128 block
+    const bool gated = a.epi.gated != 0;  // uniform: columns c and c + 64 of the wave's strip are a (gate, up) pair
+    four_times([&](auto mtc) __attribute__((always_inline)) {
+        constexpr int mt = decltype(mtc)::value;
+        four_times([&](auto ntc) __attribute__((always_inline)) {
+            constexpr int nt = decltype(ntc)::value;
+            four_times([&](auto qc) __attribute__((always_inline)) {
+                constexpr int q = decltype(qc)::value;
+                const f16& t = acc[mt][nt];
+                *reinterpret_cast<f4*>(stage + rs * kStride + 32 * nt + 8 * q + 4 * hs) =
+                    f4{t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
             });
-            // LDS operations of one wave complete in issue order: the reads below see the writes above
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            const int mrow = m0 + 128 * wm + 32 * mt;
-            if (!gated) {
+        });
+        // LDS operations of one wave complete in issue order: the reads below see the writes above
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int mrow = m0 + 128 * wm + 32 * mt;
+        if (!gated) {
 #pragma clang loop unroll(disable)
-                for (int u = 0; u < 8; ++u) {
-                    const int unit = 64 * u + lane_s, row = unit >> 4, c0 = (unit & 15) * 8;
-                    const float* src = stage + row * kStride + c0;
-                    const f4 lo = *reinterpret_cast<const f4*>(src), hi = *reinterpret_cast<const f4*>(src + 4);
-                    if (mrow + row < a.M) store_eight(a.epi, a.D, mrow + row, n0 + 128 * wn + c0, lo, hi);
-                }
-            } else {
-#pragma clang loop unroll(disable)
-                for (int u = 0; u < 4; ++u) {
-                    const int unit = 64 * u + lane_s, row = unit >> 3, c0 = (unit & 7) * 8;
-                    const float* src = stage + row * kStride + c0;
-                    const f4 glo = *reinterpret_cast<const f4*>(src), ghi = *reinterpret_cast<const f4*>(src + 4);
-                    const f4 ulo = *reinterpret_cast<const f4*>(src + 64), uhi = *reinterpret_cast<const f4*>(src + 68);
-                    if (mrow + row < a.M) store_eight_gated(a.epi, a.D, mrow + row, (n0 + 128 * wn) / 2 + c0, glo, ghi, ulo, uhi);
-                }
+            for (int u = 0; u < 8; ++u) {
+                const int unit = 64 * u + lane_s, row = unit >> 4, c0 = (unit & 15) * 8;
+                const float* src = stage + row * kStride + c0;
+                const f4 lo = *reinterpret_cast<const f4*>(src), hi = *reinterpret_cast<const f4*>(src + 4);
+                if (mrow + row < a.M) store_eight(a.epi, a.D, mrow + row, n0 + 128 * wn + c0, lo, hi);
             }
-            // the next 32 rows overwrite the block: not before these reads
-            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-            __builtin_amdgcn_wave_barrier();
-            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        });
-    } else {
-        four_times([&](auto mtc) __attribute__((always_inline)) {
-            constexpr int mt = decltype(mtc)::value;
-            const int m = m0 + 128 * wm + 32 * mt + rs;
-            if (m >= a.M) return;
-            four_times([&](auto ntc) __attribute__((always_inline)) {
-                constexpr int nt = decltype(ntc)::value;
-                four_times([&](auto qc) __attribute__((always_inline)) {
-                    constexpr int q = decltype(qc)::value;
-                    const f16& t = acc[mt][nt];
-                    const f4 v = f4{t[4 * q], t[4 * q + 1], t[4 * q + 2], t[4 * q + 3]};
-                    const int n = n0 + 128 * wn + 32 * nt + 8 * q + 4 * hs;
-                    if (a.epi.out_f32) {
-                        *reinterpret_cast<f4*>(reinterpret_cast<float*>(a.D) + (size_t)m * a.N + n) = v;
-                    } else {
-                        const h2 p0 = h2{(half_t)v[0], (half_t)v[1]};
-                        const h2 p1 = h2{(half_t)v[2], (half_t)v[3]};
-                        *reinterpret_cast<wide_u32x2*>(reinterpret_cast<half_t*>(a.D) + (size_t)m * a.N + n) =
-                            wide_u32x2{h2_to_bits(p0), h2_to_bits(p1)};
-                    }
-                });
-            });
-        });
-    }
+        } else {
+#pragma clang loop unroll(disable)
+            for (int u = 0; u < 4; ++u) {
+                const int unit = 64 * u + lane_s, row = unit >> 3, c0 = (unit & 7) * 8;
+                const float* src = stage + row * kStride + c0;
+                const f4 glo = *reinterpret_cast<const f4*>(src), ghi = *reinterpret_cast<const f4*>(src + 4);
+                const f4 ulo = *reinterpret_cast<const f4*>(src + 64), uhi = *reinterpret_cast<const f4*>(src + 68);
+                if (mrow + row < a.M) store_eight_gated(a.epi, a.D, mrow + row, (n0 + 128 * wn) / 2 + c0, glo, ghi, ulo, uhi);
+            }
+        }
+        // the next 32 rows overwrite the block: not before these reads
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    });
 }
 
 // ---------------------------------------------------------------------------------
@@ -504,9 +479,8 @@ bool wide_preferred(int m, int n, int k, unsigned tune) {
     return (double)m * n / 65536.0 >= 0.62 * 256.0 * (double)rounds;
 }
 
-template <bool EXT>
 static hipError_t wide_launch_one(const WideArgs& a, int grid, hipStream_t stream) {
-    auto kern = &w4a16_wide_kernel<EXT>;
+    auto kern = &w4a16_wide_kernel;
     static std::atomic<unsigned long long> done{0};  // the attribute is set once per device
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess) return hipErrorInvalidDevice;
@@ -535,10 +509,7 @@ int wide_launch(const void* A, int64_t lda, const void* B, const void* S, void* 
     a.mblocks = (m + 255) / 256;
     a.epi = epi;
     const int grid = (n / 256) * a.mblocks;
-    // (the plain instantiation stores 8 or 16 bytes at a time: it also needs an aligned D)
-    const bool ext = epi.gated || epi.bias || epi.residual || epi.relu2 || epi.transpose || epi.n_store != n ||
-                     epi.ldd != n || !epi.vec_ok;
-    const hipError_t e = ext ? wide_launch_one<true>(a, grid, stream) : wide_launch_one<false>(a, grid, stream);
+    const hipError_t e = wide_launch_one(a, grid, stream);
     return e == hipSuccess ? UNIQL_OK : UNIQL_E_LAUNCH;
 }
 
