@@ -13,6 +13,8 @@
 //     16 KiB, in MFMA operand order,
 //   * each wave reads 4 weight operands and 4 activation operands (16 bytes per lane each) per
 //     16 K and issues 16 MFMAs on them.
+// At the end every wave sends its quarter through LDS, 32 rows at a time, to the store code it shares with
+// the 128-column kernel (all epilogues of the layer call).
 // Against the 128 x 128 tiles of w4a16_tile_kernel (whose four waves split K and expand their own
 // weights) a weight is expanded once per 256 rows instead of once per 128, an X element is loaded
 // once per 256 columns instead of once per 128, and the weights no longer pass through the vector
