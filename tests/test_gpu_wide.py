@@ -245,3 +245,36 @@ def test_wide_kernel_random_shapes(gpu):
             g, u = v[:, :, 0].reshape(m, n // 2), v[:, :, 1].reshape(m, n // 2)
             want = g / (1 + torch.exp(-g)) * u
             assert float((y - want).abs().max()) < 1e-3 * max(1.0, float(want.abs().max())), what
+
+
+@pytest.mark.parametrize("flags", [WIDE, NARROW])
+def test_bias_and_residual_at_unaligned_addresses(gpu, flags):
+    """bias and residual are read 16 bytes at a time where their addresses allow it: a bias that starts
+    2 bytes off and a residual whose rows are 2 bytes off and an odd number of elements apart take
+    the element loads and give the same result; so does the (gate, up) form with its second bias
+    half at an odd offset"""
+    from uniql_amd import ops
+    m, k, n = 300, 256, 512
+    p = make_linear_problem(m, k, n, seed=77)
+    x, b, s = to_gpu(p, gpu)
+    ws = workspace_for(n, gpu)
+    gen = torch.Generator().manual_seed(78)
+    bias = torch.randn(n, generator=gen).half().to(gpu)
+    res = torch.randn(m, n, generator=gen).half().to(gpu)
+    want = ops.w4a16_linear(x, b, s, ws, n, k, bias=bias, residual=res, flags=flags)
+    bias_off = torch.zeros(n + 8, dtype=torch.float16, device=gpu)
+    bias_off[1:1 + n] = bias
+    res_off = torch.zeros(m * (n + 3) + 8, dtype=torch.float16, device=gpu)
+    res_view = res_off[1:1 + m * (n + 3)].view(m, n + 3)[:, :n]
+    res_view.copy_(res)
+    assert bias_off[1:1 + n].data_ptr() % 16 == 2 and res_view.stride(0) % 8 != 0
+    got = ops.w4a16_linear(x, b, s, ws, n, k, bias=bias_off[1:1 + n], residual=res_view, flags=flags)
+    assert torch.equal(got, want)
+    # gated pairs: n / 2 outputs, bias = gate biases then up biases
+    half = n // 2
+    gbias = torch.randn(2 * half, generator=gen).half().to(gpu)
+    want_g = ops.w4a16_linear(x, b, s, ws, n, k, bias=gbias, silu_mul=True, flags=flags)
+    gb_off = torch.zeros(2 * half + 8, dtype=torch.float16, device=gpu)
+    gb_off[3:3 + 2 * half] = gbias
+    got_g = ops.w4a16_linear(x, b, s, ws, n, k, bias=gb_off[3:3 + 2 * half], silu_mul=True, flags=flags)
+    assert torch.equal(got_g, want_g)
