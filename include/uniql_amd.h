@@ -33,25 +33,15 @@ enum {
     UNIQL_E_STATIC_LIMIT = -7 /* uniql_w4a16_gemm_static: the call needs more scratch than the static buffer holds */
 };
 
-/* flags of uniql_w4a16_gemm */
+/* flags of uniql_w4a16_gemm / uniql_w4a16_linear.  Bits 1, 2, 4 and 8..21 select kernels and plans
+ * for tests and measurements; they are described in uniql_amd_diag.h and are zero in production. */
 enum {
-    UNIQL_F_OUT_F32 = 1 << 0,      /* D is float32 [m, n] instead of fp16 (test hook: the value before the final rounding) */
-    UNIQL_F_FORCE_SKINNY = 1 << 1, /* use the weight-streaming kernel (default for m <= 16) whatever m is */
-    UNIQL_F_FORCE_TILED = 1 << 2,  /* use the tiled MFMA kernel (default for m > 16) whatever m is */
-    UNIQL_F_SEPARATE_ROTATION = 1 << 4, /* run a whole-row rotation as its own transform kernel into `temp` even
-                                      where the streaming kernel could apply it itself (test hook: both ways
-                                      give the same values bit for bit) */
+    UNIQL_F_OUT_F32 = 1 << 0,      /* D is float32 [m, n] instead of fp16: the value before the final rounding */
     UNIQL_F_TRANSPOSE_OUT = 1 << 3 /* the reference's output_transpose ("sequence length last",
                                       csrc/linear/marlin_gemm_kernel.cuh:574-606,1023-1026): D is [n, ldd]
                                       with D[j, i] = product[i, j]; uniql_w4a16_gemm uses ldd = m rounded up
                                       to a multiple of 8 as the reference does and leaves the padding columns
                                       untouched; uniql_w4a16_linear takes ldd >= m from the caller */
-    /* tuning hooks, 0 = choose.  Streaming kernel: bits 8..15 K-groups per wavefront,
-       bits 16..20 wavefronts per workgroup (4 or 8).
-       Tiled kernels: bits 8..15 number of K splits over workgroups, bits 16..19 row tiles of 32
-       per workgroup (1, 2 or 4: the 128-column kernel; 8: the 256 x 256 kernel for long prefill,
-       which needs n % 256 == 0, k >= 256 and grouped scales and otherwise leaves the call to the
-       128-column kernel), bits 20..21 wave quartets per workgroup (1 or 2). */
 };
 
 int uniql_abi_version(void);
@@ -63,6 +53,13 @@ const char* uniql_status_string(int code);
  * buffer needs it: a buffer allocated and zero-filled while capturing is only zero when that
  * graph replays, so it must not serve another capture or eager calls. */
 int uniql_stream_capture_id(void* stream, unsigned long long* id);
+
+/* Fills `bytes` bytes at device address `p` (both multiples of 16) with zeros, with a kernel.  No
+ * counterpart in the reference.  For the host shim's `accum` buffers: a clear that may be recorded
+ * into a graph must be a kernel node, not a memset node (memset nodes have given wrong results on
+ * replays after the first on this platform), and what an allocator's zero fill records is not
+ * under the caller's control. */
+int uniql_clear(void* p, size_t bytes, void* stream);
 
 /*
  * D[m, n] = A[m, k] . dequant(B)[k, n],  fp16 in, fp32 accumulate, fp16 out.
@@ -130,12 +127,19 @@ int uniql_w4a16_gemm(const void* A, int64_t lda, const void* B, const void* S, v
  * uniql_w4a16_gemm_static_limit(0) bytes of exchange words (4 MiB: the streaming kernel's 16-row
  * slab up to n = 32768) and uniql_w4a16_gemm_static_limit(1) bytes of temporary area (12 MiB:
  * rotated activations, the tiled kernel's partial tiles).  A call whose plan needs more of either
- * (uniql_w4a16_linear_workspace tells) returns UNIQL_E_STATIC_LIMIT and launches nothing.  The
+ * returns UNIQL_E_STATIC_LIMIT and launches nothing (the needs are those of the kernel that takes
+ * the call: at most what uniql_w4a16_linear_workspace reports, nothing at all for a long prefill
+ * on the 256 x 256 tiles).  The
  * call itself allocates and frees nothing; it enqueues one small clearing kernel for the
  * exchange words it will use, then the kernels of uniql_w4a16_gemm.
  * Every call on a GPU shares that GPU's array: calls that may overlap on one GPU (different
  * streams, or graphs replayed concurrently) race and must use uniql_w4a16_gemm with separate
  * buffers instead.
+ * Before a call is recorded into a graph, one call with the same m class (1, 2, 3..4, 5..8, 9..16,
+ * more), flags and rotation must have run eagerly on that device: the first call per device
+ * resolves the array's address (hipGetSymbolAddress) and the first launch of a kernel that uses
+ * more than 64 KiB of LDS sets a function attribute, neither of which may happen while a stream
+ * is capturing.
  */
 size_t uniql_w4a16_gemm_static_limit(int which);
 int uniql_w4a16_gemm_static(const void* A, int64_t lda, const void* B, const void* S, void* D,
@@ -201,21 +205,6 @@ int uniql_w4a16_linear(const void* A, int64_t lda, int k_in, const void* B, cons
                        int m, int n, int k, int groups,
                        int had_block, float had_scale,
                        unsigned flags, void* stream);
-
-/*
- * Measurement aid, no counterpart in the reference: launches a kernel that only READS what the
- * streaming kernel (m <= 16) of uniql_w4a16_gemm reads for this shape - every packed weight and
- * scale once, with the same grid, waves per workgroup, walk over the K groups and 16-byte loads -
- * and computes nothing.  Its duration is the floor the memory system and the launch set for that
- * plan; bench.py reports it beside the product kernel's.
- *   sink    device, uniql_w4a16_read_floor_sink_bytes(m, n, k, flags) bytes: practically never written
- *   flags   the streaming kernel's tuning fields (bits 8..15, 16..20) choose the same plan;
- *           bits 21..23: units a wave requests before it consumes the first (0 or 1: one, as the
- *           product kernel does per register set; 2 or 4: deeper)
- */
-size_t uniql_w4a16_read_floor_sink_bytes(int m, int n, int k, unsigned flags);
-int uniql_w4a16_read_floor(const void* B, const void* S, void* sink, size_t sink_bytes, int m, int n, int k,
-                           unsigned flags, void* stream);
 
 /*
  * W[k, n] fp16 = fp16_rn((code - 8) * scale), natural (un-permuted) order.

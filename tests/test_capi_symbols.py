@@ -12,10 +12,46 @@ from uniql_amd.build import LIB_PATH
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 
+HEADERS = ("uniql_amd.h", "uniql_amd_diag.h")
+
+
+def header_text():
+    text = "".join(open(os.path.join(ROOT, "include", h)).read() for h in HEADERS)
+    return re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+
+
 def header_functions():
-    text = open(os.path.join(ROOT, "include", "uniql_amd.h")).read()
-    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
-    return set(re.findall(r"\b(uniql_[a-z0-9_]+)\s*\(", text))
+    return set(re.findall(r"\b(uniql_[a-z0-9_]+)\s*\(", header_text()))
+
+
+# C parameter / return types of the headers -> the ctypes type the binding must use
+C_TO_CTYPES = {
+    "int": ctypes.c_int, "unsigned": ctypes.c_uint, "float": ctypes.c_float, "int64_t": ctypes.c_int64,
+    "size_t": ctypes.c_size_t, "const char*": ctypes.c_char_p,
+    "unsigned long long*": ctypes.POINTER(ctypes.c_ulonglong), "size_t*": ctypes.POINTER(ctypes.c_size_t),
+}
+
+
+def c_type(decl: str, is_param: bool):
+    """`const void* A` / `int64_t lda` / `size_t` -> ctypes type.  Every other pointer is passed as c_void_p."""
+    decl = decl.strip()
+    if is_param:  # drop the parameter's name
+        decl = re.sub(r"\s*\b[A-Za-z_][A-Za-z0-9_]*$", "", decl) if not decl.endswith("*") else decl
+    decl = re.sub(r"\s*\*", "*", decl).strip()
+    if decl in C_TO_CTYPES:
+        return C_TO_CTYPES[decl]
+    assert decl.endswith("*"), f"unknown C type {decl!r}"
+    return ctypes.c_void_p
+
+
+def header_prototypes():
+    """name -> (restype, [argtypes]) parsed from the declarations of the headers."""
+    protos = {}
+    for ret, name, params in re.findall(r"([A-Za-z_][A-Za-z0-9_ ]*?\**)\s*\b(uniql_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", header_text()):
+        params = params.strip()
+        args = [] if params in ("", "void") else [c_type(p, True) for p in params.split(",")]
+        protos[name] = (c_type(ret, False), args)
+    return protos
 
 
 @pytest.fixture(scope="module")
@@ -28,6 +64,33 @@ def lib():
 
 def test_header_and_binding_agree():
     assert header_functions() == set(_capi.SIGNATURES)
+
+
+def test_binding_signatures_match_the_prototypes():
+    """Return type, argument count and every argument's type of the ctypes table against the
+    prototypes as the headers spell them."""
+    protos = header_prototypes()
+    assert set(protos) == set(_capi.SIGNATURES)
+    for name, (res, args) in _capi.SIGNATURES.items():
+        want_res, want_args = protos[name]
+        assert res is want_res, f"{name}: return type {res} != {want_res}"
+        assert len(args) == len(want_args), f"{name}: {len(args)} arguments bound, {len(want_args)} declared"
+        for i, (got, want) in enumerate(zip(args, want_args)):
+            assert got is want, f"{name}: argument {i} bound as {got}, declared as {want}"
+
+
+def test_headers_compile_as_c_and_cxx(tmp_path):
+    """Both headers are plain C99 and C++17 (the boundary a cgo / JNI / pybind binding would include)."""
+    import shutil
+    import subprocess
+    src = '#include "uniql_amd_diag.h"\nint main(void) { return UNIQL_OK + UNIQL_F_FORCE_TILED * 0; }\n'
+    for compiler, std, ext in (("gcc", "-std=c99", "c"), ("g++", "-std=c++17", "cpp")):
+        if shutil.which(compiler) is None:
+            pytest.skip(f"{compiler} not available")
+        f = tmp_path / f"t.{ext}"
+        f.write_text(src)
+        subprocess.run([compiler, std, "-Wall", "-Werror", "-pedantic", "-fsyntax-only", f"-I{os.path.join(ROOT, 'include')}", str(f)],
+                       check=True)
 
 
 def test_every_declared_symbol_is_exported(lib):

@@ -1,4 +1,5 @@
-"""ctypes binding of libuniql_amd.so (the C ABI declared in include/uniql_amd.h).
+"""ctypes binding of libuniql_amd.so (the C ABI declared in include/uniql_amd.h and, for the
+test hooks and measurement aids, include/uniql_amd_diag.h).
 
 There is no fallback: if the library is missing or cannot be loaded every
 operator raises.  The library is built by `python -m uniql_amd.build`.
@@ -25,6 +26,8 @@ SIGNATURES = {
     "uniql_abi_version": (c_int, []),
     "uniql_status_string": (c_char_p, [c_int]),
     "uniql_stream_capture_id": (c_int, [c_void_p, ctypes.POINTER(ctypes.c_ulonglong)]),
+    "uniql_clear": (c_int, [c_void_p, c_size_t, c_void_p]),
+    "uniql_diag_mfma_loop": (c_int, [c_void_p, c_void_p, c_int, c_void_p]),
     "uniql_w4a16_gemm_accum_bytes": (c_size_t, [c_int, c_int, c_int]),
     "uniql_w4a16_gemm_temp_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "uniql_w4a16_gemm": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_void_p,

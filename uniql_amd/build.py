@@ -39,11 +39,7 @@ def sources() -> list[str]:
     return sorted(glob.glob(os.path.join(CSRC, "*.hip")))
 
 
-def build(verbose: bool = True) -> str:
-    """Always recompiles; returns the path of the shared library."""
-    os.makedirs(LIB_DIR, exist_ok=True)
-    tmp = LIB_PATH + ".tmp"
-    cmd = [find_hipcc(), *HIPCC_FLAGS, f"-I{INCLUDE}", f"-I{CSRC}", *sources(), "-o", tmp]
+def _run(cmd: list[str], verbose: bool) -> None:
     if verbose:
         print(" ".join(cmd), flush=True)
     proc = subprocess.run(cmd, capture_output=True, text=True)
@@ -53,6 +49,25 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError(f"hipcc failed ({proc.returncode}):\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+
+
+def build(verbose: bool = True, jobs: int | None = None) -> str:
+    """Always recompiles every source (one hipcc per file, a few at a time, into a temporary
+    directory), links, and returns the path of the shared library."""
+    import tempfile
+    from concurrent.futures import ThreadPoolExecutor
+    os.makedirs(LIB_DIR, exist_ok=True)
+    hipcc = find_hipcc()
+    compile_flags = [f for f in HIPCC_FLAGS if f != "-shared"]
+    srcs = sources()
+    jobs = jobs or max(1, min(len(srcs), (os.cpu_count() or 2) // 2, 8))
+    with tempfile.TemporaryDirectory(prefix="uniql_build_") as tmpdir:
+        objs = [os.path.join(tmpdir, os.path.basename(src)[:-4] + ".o") for src in srcs]
+        with ThreadPoolExecutor(max_workers=jobs) as pool:
+            list(pool.map(lambda so: _run([hipcc, *compile_flags, f"-I{INCLUDE}", f"-I{CSRC}", "-c", so[0], "-o", so[1]],
+                                          verbose), zip(srcs, objs)))
+        tmp = LIB_PATH + ".tmp"
+        _run([hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", *objs, "-o", tmp], verbose)
     os.replace(tmp, LIB_PATH)
     return LIB_PATH
 

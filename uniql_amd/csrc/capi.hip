@@ -3,6 +3,7 @@
 #include <mutex>
 
 #include "common.hpp"
+#include "uniql_amd_diag.h"
 
 namespace uniql {
 int stream_launch(const void* A, int64_t lda, int k_valid, const void* B, const void* S, void* D,
@@ -116,6 +117,36 @@ static size_t activation_copy_bytes(int m, int k, int k_in, int had_block, bool 
     return (rotate_first || pad_first) ? round256((size_t)m * k * sizeof(half_t)) : 0;
 }
 
+// What one layer call needs, decided in ONE place for the argument checks, the launch and the
+// entry point that brings its own scratch memory: which kernel takes the call, whether the
+// activations are copied (rotated / zero-padded) into `temp` first, and the bytes of `accum` and
+// `temp` that follow from that.  The 256 x 256 kernel needs neither buffer.
+struct LinearNeeds {
+    bool use_stream, use_wide, rotate_first, pad_first;
+    int had_mode;
+    int64_t ld_kernel;   // row stride the product kernel will see
+    size_t accum_bytes;  // rounded to 256
+    size_t act_bytes;    // copy of the activations at the start of temp (rounded to 256), or 0
+    size_t part_bytes;   // the tiled kernel's partial tiles behind it, or 0
+};
+static LinearNeeds linear_needs(int m, int n, int k, int k_in, int64_t lda, int groups, int had_block, unsigned flags) {
+    LinearNeeds q;
+    const unsigned tune = flags >> 8;
+    q.use_stream = takes_stream_kernel(m, flags);
+    q.had_mode = fused_rotation(m, k, k_in, had_block, q.use_stream, flags);
+    q.rotate_first = had_block != 0 && q.had_mode == 0;
+    // the transform kernel reads dense rows of k values: a strided or short input is first copied
+    // (and zero-padded) into the temporary buffer, then rotated there in place
+    q.pad_first = q.rotate_first ? (k_in != k || lda != k) : (k_in != k && !q.use_stream);
+    q.ld_kernel = (q.rotate_first || q.pad_first) ? (int64_t)k : lda;
+    // large M: the 256 x 256 kernel where it is the faster one and can take the call
+    q.use_wide = !q.use_stream && wide_preferred(m, n, k, tune) && wide_shape_ok(m, n, k, groups, q.ld_kernel);
+    q.accum_bytes = round256(q.use_stream ? stream_accum_bytes(m, n, k) : q.use_wide ? 0 : tile_accum_bytes(m, n, k, tune));
+    q.act_bytes = (q.rotate_first || q.pad_first) ? round256((size_t)m * k * sizeof(half_t)) : 0;
+    q.part_bytes = (q.use_stream || q.use_wide) ? 0 : tile_part_bytes(m, n, k, tune);
+    return q;
+}
+
 int uniql_w4a16_linear_workspace(int m, int n, int k, int k_in, int had_block, unsigned flags, size_t* accum_bytes,
                                  size_t* temp_bytes) {
     if (!accum_bytes || !temp_bytes) return UNIQL_E_NULL;
@@ -186,26 +217,18 @@ static int linear_impl(const void* A, int64_t lda, int k_in, const void* B, cons
         return UNIQL_E_SHAPE;
     if ((accum && !aligned16(accum)) || (temp && !aligned16(temp))) return UNIQL_E_ALIGN;
     hipStream_t st = reinterpret_cast<hipStream_t>(stream);
-    const bool use_stream = takes_stream_kernel(m, flags);
     const unsigned tune = flags >> 8;  // tuning fields, see the header
-
+    const LinearNeeds q = linear_needs(m, n, k, k_in, lda, groups, had_block, flags);
+    const bool use_stream = q.use_stream, use_wide = q.use_wide, rotate_first = q.rotate_first, pad_first = q.pad_first;
+    const int had_mode = q.had_mode;
+    const int64_t ld_kernel = q.ld_kernel;
     const void* Ain = A;
     int64_t ld = lda;
     int k_valid = k_in;
-    const int had_mode = fused_rotation(m, k, k_in, had_block, use_stream, flags);
-    const bool rotate_first = had_block != 0 && had_mode == 0;
-    // the transform kernel reads dense rows of k values: a strided or short input is first copied
-    // (and zero-padded) into the temporary buffer, then rotated there in place
-    const bool pad_first = rotate_first ? (k_in != k || lda != k) : (k_in != k && !use_stream);
-    const int64_t ld_kernel = (rotate_first || pad_first) ? (int64_t)k : lda;  // row stride the product kernel will see
-    // large M: the 256 x 256 kernel where it is the faster one and can take the call
-    const bool use_wide = !use_stream && wide_preferred(m, n, k, tune) && wide_shape_ok(m, n, k, groups, ld_kernel);
-    const size_t need_accum =
-        round256(use_stream ? stream_accum_bytes(m, n, k) : use_wide ? 0 : tile_accum_bytes(m, n, k, tune));
+    const size_t need_accum = q.accum_bytes;
     if (need_accum > 0 && (!accum || accum_bytes < need_accum)) return UNIQL_E_WORKSPACE;
     // temp: the copy of the activations, then the tiled kernel's partial tiles when it splits K
-    const size_t act_bytes = (rotate_first || pad_first) ? round256((size_t)m * k * sizeof(half_t)) : 0;
-    const size_t part_bytes = (use_stream || use_wide) ? 0 : tile_part_bytes(m, n, k, tune);
+    const size_t act_bytes = q.act_bytes, part_bytes = q.part_bytes;
     if (act_bytes + part_bytes > 0 && (!temp || temp_bytes < act_bytes + part_bytes)) return UNIQL_E_WORKSPACE;
     void* part = part_bytes ? reinterpret_cast<char*>(temp) + act_bytes : nullptr;
     // last check before the first kernel is enqueued: whether the tiled kernel can take the shape
@@ -296,11 +319,6 @@ static unsigned char* static_scratch() {
     return g_scratch_ptr[dev];
 }
 
-__global__ __launch_bounds__(256) void clear_words_kernel(u32x4* p, size_t count) {
-    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < count) p[i] = u32x4{0u, 0u, 0u, 0u};
-}
-
 size_t uniql_w4a16_gemm_static_limit(int which) {
     return which == 0 ? kStaticAccumBytes : (which == 1 ? kStaticTempBytes : 0);
 }
@@ -311,9 +329,10 @@ int uniql_w4a16_gemm_static(const void* A, int64_t lda, const void* B, const voi
     const int rc = check_linear_shape(m, n, k, groups);
     if (rc != UNIQL_OK) return rc;
     if (m == 0) return UNIQL_OK;
-    size_t need_accum = 0, need_temp = 0;
-    const int wrc = uniql_w4a16_linear_workspace(m, n, k, k, had_block, flags, &need_accum, &need_temp);
-    if (wrc != UNIQL_OK) return wrc;
+    // (the sizes of the kernel that will really take the call: a long prefill on the 256 x 256 kernel needs
+    // no scratch at all, whatever the 128-column kernel would have asked for)
+    const LinearNeeds q = linear_needs(m, n, k, k, lda, groups, had_block, flags);
+    const size_t need_accum = q.accum_bytes, need_temp = q.act_bytes + round256(q.part_bytes);
     if (need_accum > kStaticAccumBytes || need_temp > kStaticTempBytes) return UNIQL_E_STATIC_LIMIT;
     if (!A || !B || !S || !D) return UNIQL_E_NULL;
     unsigned char* base = static_scratch();
@@ -328,10 +347,8 @@ int uniql_w4a16_gemm_static(const void* A, int64_t lda, const void* B, const voi
     // shared by every call on this GPU, so the part this call uses is cleared by a small kernel
     // (a kernel, not a memset node: the call may be recorded into a graph).
     if (need_accum > 0) {
-        const size_t count = need_accum / sizeof(u32x4);
-        hipLaunchKernelGGL(clear_words_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0,
-                           reinterpret_cast<hipStream_t>(stream), reinterpret_cast<u32x4*>(base), count);
-        if (hipGetLastError() != hipSuccess) return UNIQL_E_LAUNCH;
+        const int e = uniql_clear(base, need_accum, stream);
+        if (e != UNIQL_OK) return e;
     }
     return gemm_impl(A, lda, B, S, D, workspace, workspace_len, accum, need_accum, temp, need_temp, m, n, k, groups,
                      had_block, had_scale, flags, stream, false);

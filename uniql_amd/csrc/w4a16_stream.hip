@@ -35,6 +35,8 @@
 // looks at the returned old word: whoever sees count == splits - 1 was last, owns the
 // total (old + own), stores the output and writes the word back to zero.  Integer adds
 // commute, so the result does not depend on arrival order, and nobody waits for anyone.
+#include <atomic>
+
 #include "common.hpp"
 #include "fwht_device.hpp"
 
@@ -462,14 +464,14 @@ static hipError_t launch_one(StreamArgs a, hipStream_t stream) {
     }
     auto kern = &w4a16_stream_kernel<RC, HAD, WAVES, EXT>;
     if (shmem > 64 * 1024) {
-        static bool attribute_set[64];  // per device, once per instantiation
+        static std::atomic<unsigned long long> attribute_set{0};  // a bit per device, once per instantiation
         int dev = 0;
         if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return hipErrorInvalidDevice;
-        if (!attribute_set[dev]) {
+        if (!((attribute_set.load(std::memory_order_acquire) >> dev) & 1ull)) {
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
             if (e != hipSuccess) return e;
-            attribute_set[dev] = true;
+            attribute_set.fetch_or(1ull << dev, std::memory_order_release);
         }
     }
     hipLaunchKernelGGL(kern, dim3(a.N / 128, a.splits), dim3(64 * WAVES), shmem, stream, a);

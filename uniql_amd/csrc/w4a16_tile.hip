@@ -352,6 +352,11 @@ __global__ __launch_bounds__(256 * KW, 1) void w4a16_tile_kernel(const TileArgs 
     // one again (loaded into a slot nobody reads): no branches in the loop body and constant
     // vmcnt arithmetic.
     constexpr int kDmaA = (kStageOps + 1) / 2, kDmaB = kStageOps - kDmaA;
+    // every wait below counts kStageOps loads per stage: that holds only while each half stage has an
+    // issue slot for every piece handed to it (4 MT slots, one piece every second slot from MT = 2 on)
+    constexpr int kDmaSlots = MT == 1 ? 4 : 2 * MT;
+    static_assert(kDmaA <= kDmaSlots && kDmaB <= kDmaSlots,
+                  "a half stage has fewer issue slots than LDS-DMA pieces: the vmcnt waits would lose count");
     auto group_or_last = [&](int g) __attribute__((always_inline)) { return g < g_end ? g : g_end - 1; };
     auto read_xa_one = [&](h8 (&xa)[MT], int ring, int t, int mt) __attribute__((always_inline)) {
         const uint32_t* stage = lds + ring * L::kStageDwords;
@@ -479,7 +484,7 @@ __global__ __launch_bounds__(256 * KW, 1) void w4a16_tile_kernel(const TileArgs 
                     hi += *reinterpret_cast<const f4*>(src + ww * 32 * kRedStride + 4);
                 }
                 if (split_k) {
-                    if (m < a.M) store_partial(part_mine + unit_word(mt, unit), T, lo, hi);  // rows that exist only
+                    if (m < a.M) store_partial(part_mine + unit_word(mt, unit), T, lo, hi);  // (1) rows that exist only
                 } else if (!gated) {
                     if (m < a.M) emit(m, c0, lo, hi);
                 } else {
@@ -496,16 +501,29 @@ __global__ __launch_bounds__(256 * KW, 1) void w4a16_tile_kernel(const TileArgs 
     }
     if (!split_k) return;  // uniform
 
-    // Every thread waits for its own partial stores (device-scope write-through stores) to be
-    // acknowledged before the barrier - the barrier alone does not wait for outstanding stores -
-    // so the slot is in place before thread 0 counts the workgroup in; the last workgroup reads
-    // the slots with device-scope loads.  No cache-wide write-back or invalidate is involved.
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
+    // ---- the split-K exchange: message passing with relaxed device-scope operations only -------
+    // What it relies on, step by step (the numbers are used again at the lines they govern):
+    //  (1) store_partial: relaxed agent-scope stores.  On gfx950 these are write-through (sc1)
+    //      stores that bypass the XCD's own L2, so a workgroup on another XCD can see them.
+    //  (2) s_waitcnt vmcnt(0): the counter is decremented when such a store has been ACKNOWLEDGED
+    //      by the memory side, i.e. is visible to every XCD.  A workgroup barrier alone does not
+    //      wait for outstanding stores: without this wait the arrival count below overtook the
+    //      partial tile in 8 of 130 000 randomised cases (tests/test_gpu_soak.py replays their seeds).
+    //  (3) the workgroup barrier: every thread's (2) is behind it.
+    //  (4) thread 0's relaxed agent-scope fetch_add on the tile's arrival count; nothing may move
+    //      it in front of (3) (the barrier is a compiler and hardware ordering point for it).
+    //  (5) the workgroup that completes the count reads the slots with relaxed agent-scope loads
+    //      (add_partial; sc1: they do not hit a stale line of the local L2).
+    // The language's memory model would ask for a release at (4) and an acquire before (5); at
+    // agent scope those compile to a write-back and an invalidate of the whole L2, measured at two
+    // to three times the K loop the split saves.  (2), which the ISA documents for vmcnt, stands in
+    // for the release; (5)'s cache-bypassing loads for the acquire.
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (2)
+    __syncthreads();                                   // (3)
     int* last_flag = reinterpret_cast<int*>(lds_all);
     if (tid == 0) {
         const unsigned long long old =
-            __hip_atomic_fetch_add(a.accum + tile, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            __hip_atomic_fetch_add(a.accum + tile, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // (4)
         *last_flag = (int)old == a.splits - 1;
     }
     __syncthreads();
@@ -526,7 +544,7 @@ __global__ __launch_bounds__(256 * KW, 1) void w4a16_tile_kernel(const TileArgs 
             const unsigned long long* usrc = part_tile + unit_word(mt, wunit + 8);
             f4 lo = f4{0.f, 0.f, 0.f, 0.f}, hi = lo, ulo = lo, uhi = lo;
             for (int sp = 0; sp < a.splits; ++sp) {
-                add_partial(src + (size_t)sp * kSlotWords, T, lo, hi);
+                add_partial(src + (size_t)sp * kSlotWords, T, lo, hi);  // (5)
                 if (gated) add_partial(usrc + (size_t)sp * kSlotWords, T, ulo, uhi);
             }
             if (!gated) emit(m, c0, lo, hi);

@@ -48,6 +48,23 @@
 
 namespace uniql {
 
+// ---- the K loop's load schedule, as numbers -------------------------------------------------
+// An iteration (one block of 32 K values; J = block index mod 4) issues: in its first half, when J
+// is even, the kWideXRowLoads loads of the upper rows of a pair of X blocks; in its second half one
+// load of codes, in a group's first iteration (J = 0) one load of scales, and, when J is odd, the
+// kWideXRowLoads loads of the lower rows of the next pair.  The issue sites are written with these
+// functions' constants and the waits are computed from them.
+constexpr int kWideXRowLoads = 4;
+constexpr int wide_loads_first_half(int j) { return (j & 1) == 0 ? kWideXRowLoads : 0; }
+constexpr int wide_loads_second_half(int j) { return 1 + (j == 0 ? 1 : 0) + ((j & 1) ? kWideXRowLoads : 0); }
+constexpr int wide_loads(int j) { return wide_loads_first_half(j) + wide_loads_second_half(j); }
+// loads that may still be outstanding at the barrier in the second half of iteration j (see the
+// comment at the kernel's `iteration`)
+constexpr int wide_vmcnt_at_barrier(int j) {
+    return (j & 1) ? wide_loads_second_half((j + 3) & 3)
+                   : wide_loads((j + 2) & 3) + wide_loads((j + 3) & 3) + wide_loads_first_half(j);
+}
+
 struct WideArgs {
     const u32x4* B;
     const half_t* S;
@@ -295,14 +312,20 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
     // kVm: how many loads may still be outstanding at the barrier, i.e. how many were issued after
     // the youngest one that must have landed.  Behind an odd iteration's barrier the first block
     // of the next pair is read: its upper rows were the last request of the previous iteration's
-    // first half, followed only by that iteration's codes (and scales, in a group's first
-    // iteration).  Behind an even iteration's barrier the codes of block kb+2 are fetched: the
-    // last request of iteration kb-3, followed by the 5 (6) requests each of iterations kb-2 and
-    // kb-1 and the 4 of this iteration's first half.
+    // first half, followed only by that iteration's second half (codes, and scales in a group's
+    // first iteration).  Behind an even iteration's barrier the codes of block kb+2 are fetched:
+    // the last request of iteration kb-3, followed by everything iterations kb-2 and kb-1 issue and
+    // this iteration's first half.  The counts below are the SAME constants that the issue sites
+    // are written with (loops over kXRowLoads, one load_c per iteration, load_s in iteration 0),
+    // so a load added there changes the wait here; the static_assert states the table the
+    // pipeline was validated with.
     auto iteration = [&](auto jc, auto tailc) __attribute__((always_inline)) {
         constexpr int J = decltype(jc)::value;
         constexpr bool kTail = decltype(tailc)::value != 0;
-        constexpr int kVm = J == 0 ? 14 : kTail ? 0 : J == 1 ? 2 : J == 2 ? 15 : 1;
+        constexpr int kVm = kTail && J != 0 ? 0 : wide_vmcnt_at_barrier(J);
+        static_assert(wide_vmcnt_at_barrier(0) == 14 && wide_vmcnt_at_barrier(1) == 2 && wide_vmcnt_at_barrier(2) == 15 &&
+                          wide_vmcnt_at_barrier(3) == 1,
+                      "the load schedule changed: re-derive and re-validate the waits of the K loop");
         constexpr int wbuf = J & 1, wbuf_next = (J + 1) & 1;
         // first half: K values 0..15 of block kb with operand set 0.  Meanwhile the second
         // half's operands are read and block kb+1 is expanded into the other weight buffer.
@@ -320,10 +343,9 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
             // an even iteration requests the upper rows of the pair of X blocks whose lower rows the
             // iteration before has requested (the last group's first iteration included)
             if ((J & 1) == 0 && (!kTail || J == 0)) {
-                if (i == 8) load_x(((J + 2) >> 1) & 1, 4);
-                if (i == 10) load_x(((J + 2) >> 1) & 1, 5);
-                if (i == 12) load_x(((J + 2) >> 1) & 1, 6);
-                if (i == 14) load_x(((J + 2) >> 1) & 1, 7);
+#pragma unroll
+                for (int q = 0; q < kWideXRowLoads; ++q)
+                    if (i == 8 + 2 * q) load_x(((J + 2) >> 1) & 1, kWideXRowLoads + q);
                 if (i == 15) x_next += 128;
             }
             __builtin_amdgcn_sched_barrier(0);
@@ -358,10 +380,9 @@ __global__ __launch_bounds__(256, 1) void w4a16_wide_kernel(const WideArgs a) {
                     advance3(s_issue_bytes);
                 }
                 if ((J & 1) == 1) {  // the lower rows of the pair after next, into the slot this barrier has freed
-                    if (i == 6) load_x(((J + 3) >> 1) & 1, 0);
-                    if (i == 8) load_x(((J + 3) >> 1) & 1, 1);
-                    if (i == 10) load_x(((J + 3) >> 1) & 1, 2);
-                    if (i == 12) load_x(((J + 3) >> 1) & 1, 3);
+#pragma unroll
+                    for (int q = 0; q < kWideXRowLoads; ++q)
+                        if (i == 6 + 2 * q) load_x(((J + 3) >> 1) & 1, q);
                 }
                 if (i == 14) load_c((J + 1) & 3);
                 if (i == 15) c_next += c_step;

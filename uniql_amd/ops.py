@@ -76,7 +76,10 @@ def _accumulator(device: torch.device, nbytes: int) -> torch.Tensor:
         if cbuf is None or cbuf.numel() * 8 < nbytes:
             if cbuf is not None:
                 _accum_retired.append(cbuf)
-            cbuf = torch.zeros(words, dtype=torch.int64, device=device)  # the fill is recorded in the graph
+            # cleared by the library's own kernel, so that what the graph records is a kernel node
+            # whatever this torch build's zero fill would have recorded
+            cbuf = torch.empty(words, dtype=torch.int64, device=device)
+            _capi.check(_capi.load().uniql_clear(cbuf.data_ptr(), words * 8, stream), "uniql_clear")
             _accum_in_capture[ckey] = cbuf
         return cbuf
     if buf is not None:
@@ -96,11 +99,22 @@ def reset_accumulators() -> None:
     _accum_in_capture.clear()
 
 
+_workspace_cache: dict = {}
+
+
 def _workspace(lib, m: int, n: int, k: int, k_in: int, had_block: int, flags: int):
-    """(accum bytes, temp bytes) of one layer call with these flags."""
+    """(accum bytes, temp bytes) of one layer call with these flags: a pure function of its
+    arguments, asked of the library once per distinct call shape."""
+    key = (m, n, k, k_in, had_block, flags)
+    hit = _workspace_cache.get(key)
+    if hit is not None:
+        return hit
     acc, tmp = ctypes.c_size_t(0), ctypes.c_size_t(0)
     _capi.check(lib.uniql_w4a16_linear_workspace(m, n, k, k_in, had_block, flags, ctypes.byref(acc), ctypes.byref(tmp)),
                 "uniql_w4a16_linear_workspace")
+    if len(_workspace_cache) > 4096:
+        _workspace_cache.clear()
+    _workspace_cache[key] = (acc.value, tmp.value)
     return acc.value, tmp.value
 
 
@@ -531,10 +545,42 @@ def hadamard_composite(x: torch.Tensor, scale: float, base: int) -> torch.Tensor
     return y
 
 
+class UnpinnedHadamardWarning(UserWarning):
+    """The 12N / 20N / 28N / 40N transforms use this library's own base matrices."""
+
+
+_composite_warned: set = set()
+
+
+def _composite_notice(base: int) -> None:
+    """The reference takes its 12 x 12, 20 x 20, 28 x 28 and 40 x 40 base matrices from a third-party
+    extension that is not part of its tree (quantize/hadamard_helpers.py:20-31), so the ones used
+    here (Sloane's 12, Paley 20 and 28, a doubled 20) are valid Hadamard matrices but not known
+    to be the same ones.  A model whose weights were rotated offline by the reference at such a
+    width would get a DIFFERENT online rotation here: finite, wrong outputs with no other sign.
+    Hence a warning on the first use of every base, and UNIQL_AMD_COMPOSITE_HADAMARD=error to
+    refuse instead (=quiet silences it for models rotated with this library on both sides)."""
+    import os
+    mode = os.environ.get("UNIQL_AMD_COMPOSITE_HADAMARD", "warn").lower()
+    if mode == "error":
+        raise NotImplementedError(
+            f"fast_hadamard_transform_{base}N: base matrices not pinned to the reference's (UNIQL_AMD_COMPOSITE_HADAMARD=error)")
+    if mode == "quiet" or base in _composite_warned:
+        return
+    _composite_warned.add(base)
+    import warnings
+    warnings.warn(
+        f"fast_hadamard_transform_{base}N uses this library's own {base} x {base} Hadamard matrix, which is not known to "
+        "equal the reference's: only use it where BOTH sides of a rotation (offline weights and online "
+        "activations) come from this library.  UNIQL_AMD_COMPOSITE_HADAMARD=quiet silences this, =error refuses.",
+        UnpinnedHadamardWarning, stacklevel=3)
+
+
 def composite_hadamard_variant(base: int):
     """The transform fast_hadamard_transform_{base}N(x, scale) of the reference's extension, for widths
-    base * 2^k (quantize/hadamard_helpers.py:20-31)."""
+    base * 2^k (quantize/hadamard_helpers.py:20-31).  See _composite_notice for what is not pinned."""
     def _fn(x, scale=1.0):
+        _composite_notice(base)
         return hadamard_composite(x, scale, base)
     _fn.__name__ = f"fast_hadamard_transform_{base}N"
     return _fn
