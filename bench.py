@@ -17,11 +17,20 @@ linear = K N / 2 + (K/128) N 2 + M K 2 + M N 2.  The same JSON line carries, und
 "prefill_gemm_m1024", the other half of the metric: the four linears at M = 1024 through
 the tiled MFMA kernels (TFLOP/s = 2 M K N / time, against 2.5 PFLOP/s dense fp16).
 
+The line also carries, compactly (microseconds and the fraction of the bounding peak each), every
+other size the metric is quoted on: "decode_sweep" (the four linears at M = 2, 4, 8 and the
+model's last layer 4096 -> 128256 at M = 1), "prefill_sweep" (M = 256 and 4096), "pruned_llama"
+(the four structured-pruned shapes at M = 1 and 1024, down_proj behind the fused 128-block
+rotation), "mamba2" (in_proj, the 8192-point rotation + out_proj at M = 1 and 1024, the 4-bit
+embedding gather of 2048 ids from 256000 x 4096), "secondary_kernels" (standalone transform,
+rotary kernel), "library_fp16_gemm_m1024" (torch.matmul on the same weights dequantised
+beforehand, same timing) and "mfma_only_loop" (what the matrix pipe alone sustains on such data),
+"eager_us_per_call" (the module's forward without graphs, host cost included).
+
 --sweep additionally prints (stderr) and writes (--sweep-json, default bench_sweep.json in the
-working directory) the per-shape tables: decode M in {1,2,4,8}, prefill M in {256,1024,4096},
-the pruned Llama shapes with the fused 128-block rotation, the Mamba2 shapes, the embedding
-gather, the standalone transform, the MLP front with the SiLU epilogue against the unfused
-sequence, a decoder layer's linears and glue as 5 against 12 launches, and the rotary kernel.
+working directory) the fused-layer comparisons: cache-resident decode, the MLP front with the
+SiLU epilogue against the unfused sequence, a decoder layer's linears and glue as 5 against 12
+launches, more transform and rotary sizes.
 """
 from __future__ import annotations
 
@@ -40,10 +49,23 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 LLC_BYTES = 256 << 20
-# HBM bytes per launch of the default workload (mean over the four linears) from two
+# HBM bytes per launch of the default workload (mean over the four linears) come from two
 # rocprofv3 --pmc runs of this file, FETCH_SIZE and WRITE_SIZE, each scaled by the reading for a
-# 128 MiB elementwise copy (--pmc-calibrate): factors 2.000 and 1.000.
-MEASURED_TRAFFIC_BYTES_PER_LAUNCH = 28685090
+# 128 MiB elementwise copy (--pmc-calibrate); the summary of those runs is a tracked file, and
+# the figure is read from its "traffic_bytes_per_launch = N" line at run time, so it cannot
+# outlive the profile it came from.
+TRAFFIC_PROFILE = os.path.join("profiles", "w4a16_stream_kernel_llama31_8b_decode_layer_m1_hbm_traffic.txt")
+
+
+def measured_traffic():
+    """(bytes per launch or None, source)"""
+    import re
+    try:
+        with open(os.path.join(ROOT, TRAFFIC_PROFILE)) as f:
+            m = re.search(r"traffic_bytes_per_launch\s*=\s*(\d+)", f.read())
+        return (int(m.group(1)) if m else None), TRAFFIC_PROFILE
+    except OSError:
+        return None, TRAFFIC_PROFILE
 
 LLAMA_DECODE = [("qkv", 4096, 6144), ("o_proj", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
 PRUNED = [("q_pruned", 4096, 3584, 0), ("o_pruned", 3456, 4096, 0), ("gate_up_pruned", 4096, 24320, 0),
@@ -149,8 +171,8 @@ def copies_for(bytes_per_copy):
 def cpu_baseline(budget_s=4.0):
     """The reference's CPU meaning of the layer (unpack -> un-permute -> (q-8)*s -> fp32 matmul),
     restated by the oracle, timed on this host: the four decoder-layer linears at M = 1 (the
-    workload of `value`) and o_proj at M = 1024.  Every shape runs once untimed-or-timed and then
-    as often as fits `budget_s` seconds (at most 5 times); the median is reported."""
+    workload of `value`) and o_proj at M = 1024.  Every shape runs once untimed and then at least
+    twice, as often as fits `budget_s` seconds (at most 5 times); the median is reported."""
     import torch
 
     from oracle import uniql_oracle as O
@@ -162,6 +184,7 @@ def cpu_baseline(budget_s=4.0):
         s_perm = rng.uniform(0.004, 0.02, size=(k // 128, n)).astype(np.float16)
         x = rng.standard_normal((m, k)).astype(np.float16)
         times, matmul = [], []
+        O.gemm_fp32(x, O.dequant_packed(packed, s_perm, k, n))   # untimed: first-touch page faults, thread pool start
         while True:
             t0 = time.perf_counter()
             w = O.dequant_packed(packed, s_perm, k, n)
@@ -170,7 +193,7 @@ def cpu_baseline(budget_s=4.0):
             t2 = time.perf_counter()
             times.append(t2 - t0)
             matmul.append(t2 - t1)
-            if len(times) >= 5 or sum(times) + times[-1] > budget_s:
+            if len(times) >= 5 or (len(times) >= 2 and sum(times) + times[-1] > budget_s):
                 break
         sec = float(np.median(times))
         per_shape[f"{name}_m{m}"] = {"ms": round(sec * 1e3, 1), "matmul_ms": round(float(np.median(matmul)) * 1e3, 2),
@@ -214,38 +237,13 @@ def sweep(dev, gen, out_path):
         del layer
         torch.cuda.empty_cache()
 
-    for m in (1, 2, 4, 8):
-        for name, k, n in LLAMA_DECODE:
-            bench_linear(name, k, n, m)
-    # the same launches over ONE copy of the weights: they stay in the 256 MB last-level cache
+    # the M = 1 launches over ONE copy of the weights: they stay in the 256 MB last-level cache
     # between steps, which a model of several GB never sees; reported beside the cold numbers only
     for name, k, n in LLAMA_DECODE:
         bench_linear(name + "_cache_resident", k, n, 1, copies=1)
-    for m in (256, 1024, 4096):
-        for name, k, n in LLAMA_DECODE:
-            bench_linear(name, k, n, m, steps=100)
-    for m in (1, 1024):
-        for name, k, n, hb in PRUNED + MAMBA:
-            bench_linear(name, k, (n + 255) // 256 * 256, m, hb, steps=200 if m == 1 else 100)
-
-    # the model's last layer (quantised like the others, quantize_model.py:126-143): one token's
-    # logits stream 4096 x vocabulary weights, more bytes than two decoder layers
     for name, n in (("lm_head_llama31", 128256), ("lm_head_mamba2", 256000)):
         for m in (1, 8):
             bench_linear(name, 4096, n, m, steps=60)
-
-    # embedding gather: V = 256000, D = 4096, 2048 ids
-    v, d, t = 256000, 4096, 2048
-    table = torch.randint(-2 ** 31, 2 ** 31 - 1, (v, d // 8), dtype=torch.int64, device=dev, generator=gen).to(torch.int32)
-    scales = (torch.rand(v, device=dev, generator=gen) * 0.016 + 0.004).to(torch.float16)
-    idsets = [torch.randint(0, v, (t,), device=dev, generator=gen) for _ in range(8)]
-    sec, _ = time_graphs(lambda i: ops.w4a16_embedding_lookup(idsets[i], table, scales), 8, 200, 20)
-    per = t * (d // 2 + 2 + 8 + 2 * d)
-    rows.append(dict(op="embedding_256000x4096", tokens=t, us=sec * 1e6, gbs=per / sec / 1e9,
-                     hbm_frac=per / sec / 1e9 / HBM_PEAK_GBS))
-    print("embedding 256000x4096, 2048 ids: %.2f us %.1f GB/s (%.1f%% HBM)" % (
-        sec * 1e6, per / sec / 1e9, 100 * per / sec / 1e9 / HBM_PEAK_GBS), file=sys.stderr, flush=True)
-    del table
 
     for rows_x, dim, block in ((1, 8192, 8192), (1024, 8192, 8192), (1024, 12160 + 128, 128)):
         xs = [torch.randn((rows_x, dim), device=dev, generator=gen).to(torch.float16) for _ in range(4)]
@@ -360,6 +358,108 @@ def sweep(dev, gen, out_path):
         json.dump(rows, f, indent=1)
 
 
+def eager_cost(layer, dev, calls=1000):
+    """The module's forward at M = 1 WITHOUT graphs: wall clock per call over `calls` back-to-back calls
+    (host checks, ctypes, allocation and launch included; the GPU runs behind the host), beside the
+    same kernel's time under graph replay.  The reference measures its TPOT both ways
+    (profile_model.py:502-576)."""
+    import torch
+
+    from uniql_amd.quantize.quant_linear_layers import W4A16B16O16Linear
+    mod = W4A16B16O16Linear(layer.k, layer.n, device=dev)
+    mod.weight, mod.scale = layer.weights[0]
+    x = layer.x
+    for _ in range(300):
+        mod(x)
+    torch.cuda.synchronize()
+    host, total = [], []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        for _ in range(calls):
+            mod(x)
+        host.append(time.perf_counter() - t0)   # the host's share: the loop returns before the GPU has finished
+        torch.cuda.synchronize()
+        total.append(time.perf_counter() - t0)
+    sec_k, _ = time_graphs(lambda i: mod(x), 1, 200, 40)
+    return {"shape": f"{layer.name} {layer.k}x{layer.n} m=1", "calls": calls, "repeats": 3,
+            "module_forward_host_us": round(float(np.median(host)) / calls * 1e6, 2),
+            "module_forward_wall_us": round(float(np.median(total)) / calls * 1e6, 2),
+            "same_call_graph_replay_us": round(sec_k * 1e6, 2),
+            "wall_over_kernel": round(float(np.median(total)) / calls / sec_k, 2)}
+
+
+def mfma_loop(dev, gen, iters=20000):
+    """TFLOP/s of a loop of nothing but v_mfma_f32_32x32x16_f16 on all SIMDs (uniql_diag_mfma_loop),
+    on N(0,1) operands and on zeros: the clock the chip settles at depends on the data."""
+    import ctypes
+
+    import torch
+
+    from uniql_amd import _capi
+    lib = _capi.load()
+    out = torch.empty(256 * 256, dtype=torch.float32, device=dev)
+    flops = 2.0 * 32 * 32 * 16 * 8 * iters * 1024
+    res = {"what": "256 workgroups x 4 waves, 8 independent v_mfma_f32_32x32x16_f16 per loop iteration, no loads"}
+    for label, ops_t in (("normal_data", torch.randn(512 * 8, device=dev, generator=gen).to(torch.float16)),
+                         ("zeros", torch.zeros(512 * 8, dtype=torch.float16, device=dev))):
+        stream = torch.cuda.current_stream().cuda_stream
+
+        def launch():
+            _capi.check(lib.uniql_diag_mfma_loop(ops_t.data_ptr(), out.data_ptr(), iters, stream), "uniql_diag_mfma_loop")
+        for _ in range(3):
+            launch()
+        torch.cuda.synchronize()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(5):
+            launch()
+        b.record()
+        torch.cuda.synchronize()
+        sec = a.elapsed_time(b) * 1e-3 / 5
+        res[label] = {"tflops": round(flops / sec / 1e12, 1), "frac_of_peak": round(flops / sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)}
+    return res
+
+
+def embedding_gather(dev, gen):
+    """[us, fraction of the HBM peak] of the 4-bit embedding gather: V = 256000, D = 4096, 2048 ids;
+    bytes per token: D/2 codes + scale + id + 2 D output."""
+    import torch
+
+    from uniql_amd import ops
+    v, d, t = 256000, 4096, 2048
+    table_ = torch.randint(-2 ** 31, 2 ** 31 - 1, (v, d // 8), dtype=torch.int64, device=dev, generator=gen).to(torch.int32)
+    scales = (torch.rand(v, device=dev, generator=gen) * 0.016 + 0.004).to(torch.float16)
+    idsets = [torch.randint(0, v, (t,), device=dev, generator=gen) for _ in range(8)]
+    sec, _ = time_graphs(lambda i: ops.w4a16_embedding_lookup(idsets[i], table_, scales), 8, 200, 20)
+    per = t * (d // 2 + 2 + 8 + 2 * d)
+    del table_
+    torch.cuda.empty_cache()
+    return [round(sec * 1e6, 2), round(per / sec / 1e9 / HBM_PEAK_GBS, 4)]
+
+
+def secondary(dev, gen):
+    """[us, fraction of the HBM peak] of the standalone transform (1024 rows of 8192; read + write)
+    and of the rotary kernel (1024 tokens, 32 + 8 heads of 128; q and k read and written, cos/sin read)."""
+    import torch
+
+    from uniql_amd import ops
+    out = {}
+    xs = [torch.randn((1024, 8192), device=dev, generator=gen).to(torch.float16) for _ in range(4)]
+    sec, _ = time_graphs(lambda i: ops.hadamard_blockwise(xs[i], 8192 ** -0.5, 8192), 4, 200, 20)
+    out["fwht_1024x8192"] = [round(sec * 1e6, 2), round(1024 * 8192 * 4 / sec / 1e9 / HBM_PEAK_GBS, 4)]
+    del xs
+    rows_x, d = 1024, 128
+    qs = [torch.randn((1, rows_x, 32, d), device=dev, generator=gen).to(torch.float16) for _ in range(4)]
+    ks = [torch.randn((1, rows_x, 8, d), device=dev, generator=gen).to(torch.float16) for _ in range(4)]
+    cos = torch.rand((1, rows_x, 128), device=dev, generator=gen).to(torch.float16)
+    sin = torch.rand((1, rows_x, 128), device=dev, generator=gen).to(torch.float16)
+    idx = torch.arange(d, device=dev).to(torch.uint8).repeat(8, 1)
+    sec, _ = time_graphs(lambda i: ops.rope_indices_(qs[i], ks[i], cos, sin, idx), 4, 200, 20)
+    per = rows_x * 40 * d * 2 * 2 + rows_x * 128 * 2 * 2
+    out["rope_indices_1024_tokens"] = [round(sec * 1e6, 2), round(per / sec / 1e9 / HBM_PEAK_GBS, 4)]
+    return out
+
+
 # --------------------------------------------------------------------------------------
 def main():
     ap = argparse.ArgumentParser()
@@ -394,6 +494,8 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    from uniql_amd import ops
+
     m = 1
     step_bytes = sum(linear_bytes(m, k, n) for _, k, n in LLAMA_DECODE)
     weight_bytes = sum(k * n // 2 for _, k, n in LLAMA_DECODE)
@@ -407,6 +509,7 @@ def main():
     launches = len(layers)
     gbs = step_bytes / sec_per_step / 1e9
     kernel_us = sec_per_step / launches * 1e6
+    traffic, traffic_source = measured_traffic()
     result = {
         "metric": "W4A16 GEMV GB/s at M=1 (Llama-3.1-8B decoder-layer linears)", "value": round(gbs, 2),
         "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -416,13 +519,13 @@ def main():
                    "m": m, "group_size": 128, "weight_copies_rotated": copies, "launch": "hip_graph",
                    "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "wall_ms_per_step": round(wall_per_step * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": MEASURED_TRAFFIC_BYTES_PER_LAUNCH,
-                     "kernel": "w4a16_stream_kernel<RC=1,HAD=false> (all four launches of a step)", "launches_per_step": launches,
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
+                     "kernel": "w4a16_stream_kernel<RC=1, HAD=0, WAVES=4, EXT=false> (all four launches of a step)",
+                     "launches_per_step": launches,
                      "avg_launch_us": round(kernel_us, 3), "bytes_per_launch": step_bytes // launches},
     }
     # what the memory system and the launch alone allow: the kernel that only reads the same bytes with the
     # same plan (uniql_w4a16_read_floor), per linear, beside the product kernel timed the same way
-    from uniql_amd import ops
     floor = {}
     for layer in layers:
         def product(i, layer=layer):
@@ -442,21 +545,60 @@ def main():
     tiny = torch.zeros(64, device=dev)
     sec_e, _ = time_graphs(lambda i: tiny.fill_(1.0), 1, 400, 40)
     result["config"]["empty_kernel_us_per_graph_node"] = round(sec_e * 1e6, 2)
+    result["eager_us_per_call"] = eager_cost(layers[1], dev)
     del layers
     torch.cuda.empty_cache()
 
-    # second half of the metric: the same four linears at M = 1024 through the tiled MFMA kernel
+    def one_linear(name, k, n, rows, had_block=0, steps=None):
+        """[us, fraction of the bounding peak]: HBM for up to 16 rows, dense fp16 MFMA beyond"""
+        cps = copies_for(k * n // 2) if rows <= 64 else 2
+        layer = Layer(name, k, n, rows, cps, dev, gen, had_block)
+        sec, _ = time_graphs(lambda i: layer.run(i), cps, steps or (120 if rows <= 64 else 60), 40)
+        del layer
+        torch.cuda.empty_cache()
+        if rows <= 16:
+            return sec, linear_bytes(rows, k, n) / sec / 1e9 / HBM_PEAK_GBS
+        return sec, linear_flops(rows, k, n) / sec / 1e12 / MFMA_F16_PEAK_TFLOPS
+
+    def table(shapes, rows_list):
+        out = {}
+        for rows in rows_list:
+            row, tot = {}, 0.0
+            for name, k, n, *rest in shapes:
+                sec, frac = one_linear(name, k, (n + 255) // 256 * 256, rows, rest[0] if rest else 0)
+                row[name] = [round(sec * 1e6, 2), round(frac, 4)]
+                tot += sec
+            row["sum_us"] = round(tot * 1e6, 2)
+            out[f"m{rows}"] = row
+        return out
+
+    # the decode sweep's other columns and the model's last layer (quantised like the rest,
+    # quantize_model.py:126-143): [us, fraction of the HBM peak]
+    result["decode_sweep"] = table(LLAMA_DECODE, (2, 4, 8))
+    sec, frac = one_linear("lm_head", 4096, 128256, 1, steps=60)
+    result["decode_sweep"]["lm_head_llama31_4096x128256_m1"] = [round(sec * 1e6, 2), round(frac, 4)]
+
+    # second half of the metric: the same four linears at M = 1024 through the tiled MFMA kernels,
+    # and beside them the library's fp16 GEMM on the same weights dequantised beforehand
     pm = 1024
     per_shape, tot_flops, tot_sec = {}, 0.0, 0.0
+    lib_shape, lib_sec = {}, 0.0
     for name, k, n in LLAMA_DECODE:
         layer = Layer(name, k, n, pm, 2, dev, gen)
-        # the clocks of a chip that was idle take a few milliseconds to settle: 40 untimed steps first
         sec, _ = time_graphs(lambda i: layer.run(i), 2, 100, 40)
         fl = linear_flops(pm, k, n)
         per_shape[name] = {"us": round(sec * 1e6, 2), "tflops": round(fl / sec / 1e12, 1)}
         tot_flops += fl
         tot_sec += sec
-        del layer
+        dense = [ops.w4a16_dequant(b, s_, n, k) for b, s_ in layer.weights]   # [k, n] fp16, natural order
+        x = layer.x
+        ref = torch.matmul(x, dense[0])
+        err = (ref.float() - layer.run(0).float()).abs().max().item()
+        sec_l, _ = time_graphs(lambda i: torch.matmul(x, dense[i % 2]), 2, 100, 40)
+        lib_shape[name] = {"us": round(sec_l * 1e6, 2), "tflops": round(fl / sec_l / 1e12, 1),
+                           "ours_over_library": round(sec_l / sec, 3), "max_abs_diff": round(err, 4)}
+        lib_sec += sec_l
+        del layer, dense
         torch.cuda.empty_cache()
     result["prefill_gemm_m1024"] = {
         "metric": "W4A16 prefill GEMM TFLOP/s at M=1024 (same four linears)", "value": round(tot_flops / tot_sec / 1e12, 1),
@@ -465,6 +607,20 @@ def main():
                      "unit": "TFLOP/s", "frac": round(tot_flops / tot_sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                      "kernel": "w4a16_wide_kernel (256 x 256 tiles) for gate_up, w4a16_tile_kernel<MT> (MT = 4, or 2 for the "
                                "6144-wide qkv) for the other three"}}
+    result["library_fp16_gemm_m1024"] = {
+        "what": "torch.matmul(x[1024, k] fp16, w[k, n] fp16) on the same weights dequantised beforehand (its dequantisation "
+                "pass not counted), same graph timing",
+        "value": round(tot_flops / lib_sec / 1e12, 1), "unit": "TFLOP/s", "us_per_layer": round(lib_sec * 1e6, 2),
+        "frac_of_peak": round(tot_flops / lib_sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4), "per_linear": lib_shape}
+    result["mfma_only_loop"] = mfma_loop(dev, gen)
+    # [us, fraction of the dense fp16 MFMA peak]
+    result["prefill_sweep"] = table(LLAMA_DECODE, (256, 4096))
+    # configs[3]: structured-pruned Llama (widths padded to multiples of 256 as the module pads them);
+    # down_proj behind the fused 128-block rotation.  configs[4]: the Mamba2 block.
+    result["pruned_llama"] = table(PRUNED, (1, 1024))
+    result["mamba2"] = table(MAMBA, (1, 1024))
+    result["mamba2"]["embedding_256000x4096_2048ids"] = embedding_gather(dev, gen)
+    result["secondary_kernels"] = secondary(dev, gen)
     if args.sweep:
         sweep(dev, gen, args.sweep_json)
     if not args.no_cpu:

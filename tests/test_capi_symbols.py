@@ -134,6 +134,26 @@ def test_host_only_entry_points(lib):
     assert lib.uniql_w4a16_read_floor(None, None, None, 0, 1, 4096, 4096, 0, None) == -1
 
 
+def test_static_entry_uses_the_needs_of_the_kernel_that_takes_the_call(lib):
+    """uniql_w4a16_gemm_static sizes its scratch with the same decision as the launch: a prefill that
+    the 256 x 256 kernel takes needs none (and passes the limit check whatever the 128-column
+    kernel would have asked for), the same shape forced onto the 128-column kernel with K splits
+    needs partial tiles beyond the static area and is refused before the pointers are looked at."""
+    st = lib.uniql_w4a16_gemm_static
+    acc, tmp = ctypes.c_size_t(0), ctypes.c_size_t(0)
+    split4_tile128 = (4 << 8) | (4 << 16)     # four K splits, 128-row tiles of the 128-column kernel
+    wide = 8 << 16                            # the 256 x 256 kernel
+    m, n, k = 1024, 4096, 4096
+    assert lib.uniql_w4a16_linear_workspace(m, n, k, k, 0, split4_tile128, ctypes.byref(acc), ctypes.byref(tmp)) == 0
+    assert tmp.value == 4 * m * n * 4 > lib.uniql_w4a16_gemm_static_limit(1)
+    assert st(None, k, None, None, None, None, 0, m, n, k, k // 128, 0, 1.0, split4_tile128, None) == -7
+    assert st(None, k, None, None, None, None, 0, m, n, k, k // 128, 0, 1.0, wide, None) == -1      # no scratch needed: next check
+    # per-column scales cannot take the 256 x 256 kernel: the call falls to the 128-column kernel's own plan
+    assert st(None, k, None, None, None, None, 0, m, n, k, 1, 0, 1.0, wide, None) == -1
+    # the default plan of a long, wide prefill: the 256 x 256 kernel, nothing to clear, nothing to refuse
+    assert st(None, 4096, None, None, None, None, 0, 4096, 28672, 4096, 32, 0, 1.0, 0, None) == -1
+
+
 def test_argument_checks_need_no_gpu(lib):
     """Shape errors are reported before anything touches the device."""
     f = lib.uniql_w4a16_gemm

@@ -234,6 +234,32 @@ def test_nan_propagates_with_and_without_k_split(gpu, m):
     assert np.isnan(y16[m - 1]).all()
 
 
+def test_infinite_partial_sums_with_and_without_k_split(gpu):
+    """What the header documents for partial sums beyond the accumulator words' range, pinned:
+    an infinite activation gives an infinite fp16 result of the right sign with and without a K
+    split (a partial sum clamped to +-2^18 is still beyond fp16's 65504); with fp32 output the
+    launch that splits K shows the clamp (a finite value of at least 2^18) where the launch
+    that does not split shows inf; +inf and -inf that meet from different workgroups cancel to
+    a finite value when K is split and give NaN when it is not."""
+    m, k, n = 2, 4096, 512
+    p = make_linear_problem(m, k, n, seed=77)
+    p["q"][:] = 15                      # every weight +7 s > 0: the sign of a column's sum is the activation's
+    p["packed"] = O.pack_weights(p["q"])
+    p["x"][:] = np.float16(0.001)
+    p["x"][0, 100] = np.inf             # row 0: +inf in the first workgroup's K range
+    p["x"][1, 100] = np.inf             # row 1: +inf there and -inf in the last workgroup's
+    p["x"][1, 4000] = -np.inf
+    whole_plan = (8 << 8) | (4 << 16)   # 4 waves x 8 groups: one workgroup per strip, no exchange
+    y_split, y_whole = run_gemm(p, gpu), run_gemm(p, gpu, flags=whole_plan)
+    for y in (y_split, y_whole):
+        assert np.isposinf(y[0]).all()
+    assert np.isnan(y_whole[1]).all()               # inf - inf inside one workgroup's fp32 sum
+    assert np.isfinite(y_split[1]).all()            # the documented difference: clamped partial sums cancel
+    f_split, f_whole = run_gemm(p, gpu, out_f32=True), run_gemm(p, gpu, out_f32=True, flags=whole_plan)
+    assert np.isposinf(f_whole[0]).all()
+    assert np.isfinite(f_split[0]).all() and (f_split[0] >= 2.0 ** 18).all()
+
+
 def test_row_stride(gpu):
     """A may be a row-strided view (lda > k)."""
     from uniql_amd import ops

@@ -19,7 +19,8 @@ import torch
 from . import _capi
 
 __all__ = [
-    "w4a16o16_gemm", "w4a16_gemm_ex", "w4a16_gemm_static", "w4a16_linear", "w4a16_dequant", "w4a16_embedding_lookup",
+    "w4a16o16_gemm", "w4a16_gemm_ex", "w4a16_gemm_static", "w4a16_linear", "prepare_linear", "linear_prepared",
+    "w4a16_dequant", "w4a16_embedding_lookup",
     "fast_hadamard_transform", "hadamard_blockwise", "hadamard_composite", "composite_hadamard_variant",
     "w4a16_read_floor", "w4a16_quantize", "w4a16_pack", "w4a16_unpack", "w4_embedding_quantize", "rope_indices_",
 ]
@@ -62,8 +63,9 @@ def _capture_id(stream_ptr: int) -> int:
     return out.value
 
 
-def _accumulator(device: torch.device, nbytes: int) -> torch.Tensor:
-    stream = _stream_ptr(device)
+def _accumulator(device: torch.device, nbytes: int, stream: int | None = None) -> torch.Tensor:
+    if stream is None:
+        stream = _stream_ptr(device)
     key = (device.index, stream)
     buf = _accum_cache.get(key)
     if buf is not None and buf.numel() * 8 >= nbytes:
@@ -206,6 +208,112 @@ def w4a16_gemm_static(A: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspa
     return out
 
 
+class PreparedLinear:
+    """What a layer call needs that does not change from call to call, validated once
+    (prepare_linear): the packed tensors, their addresses and sizes, bias, rotation, epilogue.
+    The tensors are held so that the addresses stay valid."""
+    __slots__ = ("B", "s", "workspace", "bias", "b_ptr", "s_ptr", "ws_ptr", "ws_len", "bias_ptr", "size_n", "size_k",
+                 "n_out", "groups", "had_block", "had_scale", "silu_mul", "dev", "needs")
+
+
+def prepare_linear(B: torch.Tensor, s: torch.Tensor, workspace: torch.Tensor, size_n: int, size_k: int, *,
+                   out_features: int | None = None, bias: torch.Tensor | None = None, silu_mul: bool = False,
+                   had_block: int = 0, had_scale: float = 1.0) -> PreparedLinear:
+    """Every check of w4a16_linear that concerns the layer and not the activations."""
+    for t, name in ((B, "B"), (s, "s"), (workspace, "workspace")):
+        _require_gpu(t, name)
+    if s.dtype != torch.float16:
+        raise RuntimeError("x and s must be float16")
+    if B.dtype != torch.int32 or workspace.dtype != torch.int32:
+        raise RuntimeError("B and workspace must be int32")
+    if not (B.is_contiguous() and s.is_contiguous() and workspace.is_contiguous()):
+        raise RuntimeError("B, s and workspace must be contiguous")
+    if tuple(B.shape) != (size_k // 16, 2 * size_n) or s.dim() != 2 or s.shape[1] != size_n:
+        raise RuntimeError("B / s shapes do not match size_k, size_n")
+    n_max = size_n // 2 if silu_mul else size_n
+    n_out = n_max if out_features is None else int(out_features)
+    if not 0 < n_out <= n_max:
+        raise RuntimeError(f"out_features={n_out} does not fit the packed width {n_max}")
+    if bias is not None:
+        _require_gpu(bias, "bias")
+        if bias.dtype != torch.float16 or not bias.is_contiguous() or bias.numel() != (2 if silu_mul else 1) * n_out:
+            raise RuntimeError("bias must be contiguous float16 with one entry per output column")
+    p = PreparedLinear()
+    p.B, p.s, p.workspace, p.bias = B, s, workspace, bias
+    p.b_ptr, p.s_ptr, p.ws_ptr, p.ws_len = B.data_ptr(), s.data_ptr(), workspace.data_ptr(), workspace.numel()
+    p.bias_ptr = bias.data_ptr() if bias is not None else None
+    p.size_n, p.size_k, p.n_out, p.groups = int(size_n), int(size_k), n_out, s.shape[0]
+    p.had_block, p.had_scale, p.silu_mul = int(had_block), float(had_scale), bool(silu_mul)
+    p.dev = B.device
+    p.needs = {}   # (m, k_in, flags) -> (accum bytes, temp bytes)
+    return p
+
+
+def linear_prepared(p: PreparedLinear, x: torch.Tensor, *, residual: torch.Tensor | None = None, relu2: bool = False,
+                    out_f32: bool = False, out: torch.Tensor | None = None, flags: int = 0) -> torch.Tensor:
+    """The per-call half of w4a16_linear: checks on the activations (and residual / out), the
+    output's allocation, one call into the library."""
+    if not x.is_cuda:
+        raise RuntimeError("x must be a GPU tensor (this package has no CPU path)")
+    if x.dtype != torch.float16:
+        raise RuntimeError("x and s must be float16")
+    if x.dim() != 2 or x.stride(1) != 1:
+        raise RuntimeError("x must be 2-D with unit stride along K")
+    m, k_in = x.shape
+    size_k, n_out = p.size_k, p.n_out
+    if not (size_k - 128 < k_in <= size_k):
+        raise RuntimeError(f"x has {k_in} columns, the packed weights cover {size_k}")
+    if p.silu_mul and relu2:
+        raise RuntimeError("silu_mul and relu2 are different epilogues: choose one")
+    res_ptr, ldr = None, 0
+    if residual is not None:
+        _require_gpu(residual, "residual")
+        if p.silu_mul or relu2:
+            raise RuntimeError("a residual cannot be combined with an activation epilogue")
+        if residual.dtype != torch.float16 or tuple(residual.shape) != (m, n_out) or residual.stride(1) != 1:
+            raise RuntimeError("residual must be float16 [m, out_features] with unit inner stride")
+        res_ptr, ldr = residual.data_ptr(), (residual.stride(0) if m > 1 else n_out)
+    x_ptr = x.data_ptr()
+    if k_in % 8 or (m > 1 and x.stride(0) % 8) or x_ptr % 16:
+        # rare: rows that cannot be read in 16-byte pieces are copied (and padded) here
+        x = torch.nn.functional.pad(x, (0, size_k - k_in))
+        k_in = size_k
+        x_ptr = x.data_ptr()
+    lib = _capi.load()
+    dev = x.device
+    out_dtype = torch.float32 if out_f32 else torch.float16
+    with _device_guard(dev):
+        if out is None:
+            out = torch.empty((m, n_out), dtype=out_dtype, device=dev)
+        elif out.dtype != out_dtype or tuple(out.shape) != (m, n_out) or out.stride(1) != 1 or out.device != dev:
+            raise RuntimeError("out must be a [m, out_features] view with unit inner stride on x's device")
+        if m == 0:
+            return out
+        if out_f32:
+            flags |= _capi.F_OUT_F32
+        key = (m, k_in, flags)
+        need = p.needs.get(key)
+        if need is None:
+            need = p.needs[key] = _workspace(lib, m, p.size_n, size_k, k_in, p.had_block, flags)
+        need_acc, need_tmp = need
+        stream = _stream_ptr(dev)
+        accum = _accumulator(dev, need_acc, stream) if need_acc else None
+        temp = torch.empty(need_tmp, dtype=torch.uint8, device=dev) if need_tmp else None
+        lda = x.stride(0) if m > 1 else max(k_in + (-k_in) % 8, 8)
+        ldd = out.stride(0) if m > 1 else n_out
+        code = lib.uniql_w4a16_linear(
+            x_ptr, lda, k_in, p.b_ptr, p.s_ptr, p.bias_ptr, res_ptr, ldr,
+            out.data_ptr(), ldd, n_out,
+            _capi.EPI_SILU_MUL if p.silu_mul else (_capi.EPI_RELU2 if relu2 else _capi.EPI_NONE),
+            p.ws_ptr, p.ws_len,
+            accum.data_ptr() if accum is not None else None, accum.numel() * 8 if accum is not None else 0,
+            temp.data_ptr() if temp is not None else None, need_tmp,
+            m, p.size_n, size_k, p.groups, p.had_block, p.had_scale, flags, stream)
+    if code:
+        _capi.check(code, "uniql_w4a16_linear")
+    return out
+
+
 def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: torch.Tensor, size_n: int,
                  size_k: int, *, out_features: int | None = None, bias: torch.Tensor | None = None,
                  residual: torch.Tensor | None = None, silu_mul: bool = False, relu2: bool = False,
@@ -221,71 +329,14 @@ def w4a16_linear(x: torch.Tensor, B: torch.Tensor, s: torch.Tensor, workspace: t
     With `relu2` the result is relu(y)^2 of the (biased) output y, the un-gated MLP front of the
     squared-ReLU models.
     `out`: optional destination, a 2-D view with unit inner stride (for example a column range
-    of a larger buffer)."""
-    for t, name in ((x, "x"), (B, "B"), (s, "s"), (workspace, "workspace")):
-        _require_gpu(t, name)
-    if x.dtype != torch.float16 or s.dtype != torch.float16:
-        raise RuntimeError("x and s must be float16")
-    if B.dtype != torch.int32 or workspace.dtype != torch.int32:
-        raise RuntimeError("B and workspace must be int32")
-    if x.dim() != 2 or x.stride(1) != 1:
-        raise RuntimeError("x must be 2-D with unit stride along K")
-    m, k_in = x.shape
-    if not (size_k - 128 < k_in <= size_k):
-        raise RuntimeError(f"x has {k_in} columns, the packed weights cover {size_k}")
-    if not (B.is_contiguous() and s.is_contiguous() and workspace.is_contiguous()):
-        raise RuntimeError("B, s and workspace must be contiguous")
-    if tuple(B.shape) != (size_k // 16, 2 * size_n) or s.dim() != 2 or s.shape[1] != size_n:
-        raise RuntimeError("B / s shapes do not match size_k, size_n")
-    if silu_mul and relu2:
-        raise RuntimeError("silu_mul and relu2 are different epilogues: choose one")
-    n_max = size_n // 2 if silu_mul else size_n
-    n_out = n_max if out_features is None else int(out_features)
-    if not 0 < n_out <= n_max:
-        raise RuntimeError(f"out_features={n_out} does not fit the packed width {n_max}")
-    if bias is not None:
-        _require_gpu(bias, "bias")
-        if bias.dtype != torch.float16 or not bias.is_contiguous() or bias.numel() != (2 if silu_mul else 1) * n_out:
-            raise RuntimeError("bias must be contiguous float16 with one entry per output column")
-    if residual is not None:
-        _require_gpu(residual, "residual")
-        if silu_mul or relu2:
-            raise RuntimeError("a residual cannot be combined with an activation epilogue")
-        if residual.dtype != torch.float16 or tuple(residual.shape) != (m, n_out) or residual.stride(1) != 1:
-            raise RuntimeError("residual must be float16 [m, out_features] with unit inner stride")
-    if k_in % 8 or (m > 1 and x.stride(0) % 8) or x.data_ptr() % 16:
-        # rare: rows that cannot be read in 16-byte pieces are copied (and padded) here
-        x = torch.nn.functional.pad(x, (0, size_k - k_in))
-        k_in = size_k
-    lib = _capi.load()
-    dev = x.device
-    out_dtype = torch.float32 if out_f32 else torch.float16
-    with _device_guard(dev):
-        if out is None:
-            out = torch.empty((m, n_out), dtype=out_dtype, device=dev)
-        elif out.dtype != out_dtype or tuple(out.shape) != (m, n_out) or out.stride(1) != 1 or out.device != dev:
-            raise RuntimeError("out must be a [m, out_features] view with unit inner stride on x's device")
-        if m == 0:
-            return out
-        if out_f32:
-            flags |= _capi.F_OUT_F32
-        need_acc, need_tmp = _workspace(lib, m, size_n, size_k, k_in, had_block, flags)
-        accum = _accumulator(dev, need_acc) if need_acc else None
-        temp = torch.empty(need_tmp, dtype=torch.uint8, device=dev) if need_tmp else None
-        lda = x.stride(0) if m > 1 else max(k_in + (-k_in) % 8, 8)
-        ldd = out.stride(0) if m > 1 else n_out
-        code = lib.uniql_w4a16_linear(
-            x.data_ptr(), lda, k_in, B.data_ptr(), s.data_ptr(), bias.data_ptr() if bias is not None else None,
-            residual.data_ptr() if residual is not None else None,
-            (residual.stride(0) if m > 1 else n_out) if residual is not None else 0,
-            out.data_ptr(), ldd, n_out,
-            _capi.EPI_SILU_MUL if silu_mul else (_capi.EPI_RELU2 if relu2 else _capi.EPI_NONE),
-            workspace.data_ptr(), workspace.numel(),
-            accum.data_ptr() if accum is not None else None, accum.numel() * 8 if accum is not None else 0,
-            temp.data_ptr() if temp is not None else None, need_tmp,
-            m, size_n, size_k, s.shape[0], had_block, float(had_scale), flags, _stream_ptr(dev))
-    _capi.check(code, "uniql_w4a16_linear")
-    return out
+    of a larger buffer).
+    A caller that runs the same layer again and again validates it once with prepare_linear and
+    calls linear_prepared (the module classes do): the checks on the packed tensors are about a
+    third of this call's host time."""
+    _require_gpu(x, "x")
+    p = prepare_linear(B, s, workspace, size_n, size_k, out_features=out_features, bias=bias, silu_mul=silu_mul,
+                       had_block=had_block, had_scale=had_scale)
+    return linear_prepared(p, x, residual=residual, relu2=relu2, out_f32=out_f32, out=out, flags=flags)
 
 
 def w4a16o16_gemm(A, B, s, workspace, size_m, size_n, size_k, output_transpose=False,

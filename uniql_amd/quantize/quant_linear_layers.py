@@ -103,16 +103,29 @@ class W4A16B16O16Linear(nn.Module):
         of the un-gated MLP (nemotron_h_qblocks.py:588: act_fn(up_proj(x))) to the result."""
         if activation not in (None, "relu2"):
             raise ValueError(f"unsupported activation {activation!r} (None or 'relu2')")
-        lead = x.shape[:-1]
-        x2 = x.reshape(-1, x.shape[-1])
+        x2 = x if x.dim() == 2 else x.reshape(-1, x.shape[-1])
         if x2.stride(-1) != 1:
             x2 = x2.contiguous()
-        y = ops.w4a16_linear(x2, self.weight, self.scale, self.workspace, self.size_n, self.size_k,
-                             out_features=self.out_features, bias=None if self.bias is None else self.bias.data,
-                             residual=None if residual is None else residual.reshape(-1, self.out_features),
-                             relu2=activation == "relu2",
-                             had_block=self.had_block, had_scale=self.had_scale)
-        return y.view(*lead, self.out_features)
+        y = ops.linear_prepared(self._prepared(), x2,
+                                residual=None if residual is None else residual.reshape(-1, self.out_features),
+                                relu2=activation == "relu2")
+        return y if x.dim() == 2 else y.view(*x.shape[:-1], self.out_features)
+
+    def _prepared(self):
+        """The layer's side of the call, validated once and kept until a buffer is replaced
+        (load_state_dict copies in place and keeps it; .to(device) or an assignment does not)."""
+        buffers = self._buffers
+        weight, scale, workspace = buffers["weight"], buffers["scale"], buffers["workspace"]
+        bias = self.bias
+        key = (weight.data_ptr(), scale.data_ptr(), workspace.data_ptr(), None if bias is None else bias.data_ptr(),
+               self.had_block, self.had_scale, self.size_n, self.size_k, self.out_features)
+        cached = self.__dict__.get("_prep")
+        if cached is None or cached[0] != key:
+            prep = ops.prepare_linear(weight, scale, workspace, self.size_n, self.size_k, out_features=self.out_features,
+                                      bias=None if bias is None else bias.data, had_block=self.had_block,
+                                      had_scale=self.had_scale)
+            cached = self.__dict__["_prep"] = (key, prep)
+        return cached[1]
 
     def __repr__(self):
         return (f"W4A16B16O16Linear(in_features={self.in_features}, out_features={self.out_features}, "
