@@ -469,6 +469,11 @@ def main():
     ap.add_argument("--sweep", action="store_true")
     ap.add_argument("--sweep-json", default="bench_sweep.json", help="where --sweep writes its table")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--sections", default="all",
+                    help="comma-separated parts to run behind the headline step (default all): floor (per-linear product "
+                         "and read-floor times, empty kernel, eager cost), decode_sweep, prefill (M = 1024, library GEMM, "
+                         "MFMA-only loop), prefill_sweep, models (pruned Llama, Mamba2, embedding), secondary (transform, "
+                         "rotary), or none.  Profiler runs name the parts whose kernels they summarise.")
     ap.add_argument("--pmc-calibrate", action="store_true",
                     help="also launch three plain elementwise copies of 128 MiB (read 128 MiB, write 128 MiB each) "
                          "before the timed region: the known-size kernel a rocprofv3 --pmc run scales its "
@@ -495,6 +500,11 @@ def main():
         del src, dst
 
     from uniql_amd import ops
+    known = ("floor", "decode_sweep", "prefill", "prefill_sweep", "models", "secondary")
+    want = set(known) if args.sections == "all" else set(x for x in args.sections.split(",") if x and x != "none")
+    if not want <= set(known):
+        print(f"--sections: unknown part(s) {sorted(want - set(known))}; known: {known}", file=sys.stderr)
+        sys.exit(2)
 
     m = 1
     step_bytes = sum(linear_bytes(m, k, n) for _, k, n in LLAMA_DECODE)
@@ -527,7 +537,7 @@ def main():
     # what the memory system and the launch alone allow: the kernel that only reads the same bytes with the
     # same plan (uniql_w4a16_read_floor), per linear, beside the product kernel timed the same way
     floor = {}
-    for layer in layers:
+    for layer in (layers if "floor" in want else []):
         def product(i, layer=layer):
             return layer.run(i)
 
@@ -539,13 +549,14 @@ def main():
         floor[layer.name] = {"kernel_us": round(sec_k * 1e6, 2), "read_floor_us": round(sec_f * 1e6, 2),
                              "gbs": round(linear_bytes(m, layer.k, layer.n) / sec_k / 1e9, 1),
                              "hbm_frac": round(linear_bytes(m, layer.k, layer.n) / sec_k / 1e9 / HBM_PEAK_GBS, 4)}
-    result["config"]["per_linear"] = floor
-    result["config"]["read_floor_us_per_step"] = round(sum(v["read_floor_us"] for v in floor.values()), 2)
-    # what one node of a replayed graph costs when its kernel does nothing (one workgroup fills 64 floats)
-    tiny = torch.zeros(64, device=dev)
-    sec_e, _ = time_graphs(lambda i: tiny.fill_(1.0), 1, 400, 40)
-    result["config"]["empty_kernel_us_per_graph_node"] = round(sec_e * 1e6, 2)
-    result["eager_us_per_call"] = eager_cost(layers[1], dev)
+    if "floor" in want:
+        result["config"]["per_linear"] = floor
+        result["config"]["read_floor_us_per_step"] = round(sum(v["read_floor_us"] for v in floor.values()), 2)
+        # what one node of a replayed graph costs when its kernel does nothing (one workgroup fills 64 floats)
+        tiny = torch.zeros(64, device=dev)
+        sec_e, _ = time_graphs(lambda i: tiny.fill_(1.0), 1, 400, 40)
+        result["config"]["empty_kernel_us_per_graph_node"] = round(sec_e * 1e6, 2)
+        result["eager_us_per_call"] = eager_cost(layers[1], dev)
     del layers
     torch.cuda.empty_cache()
 
@@ -574,16 +585,17 @@ def main():
 
     # the decode sweep's other columns and the model's last layer (quantised like the rest,
     # quantize_model.py:126-143): [us, fraction of the HBM peak]
-    result["decode_sweep"] = table(LLAMA_DECODE, (2, 4, 8))
-    sec, frac = one_linear("lm_head", 4096, 128256, 1, steps=60)
-    result["decode_sweep"]["lm_head_llama31_4096x128256_m1"] = [round(sec * 1e6, 2), round(frac, 4)]
+    if "decode_sweep" in want:
+        result["decode_sweep"] = table(LLAMA_DECODE, (2, 4, 8))
+        sec, frac = one_linear("lm_head", 4096, 128256, 1, steps=60)
+        result["decode_sweep"]["lm_head_llama31_4096x128256_m1"] = [round(sec * 1e6, 2), round(frac, 4)]
 
     # second half of the metric: the same four linears at M = 1024 through the tiled MFMA kernels,
     # and beside them the library's fp16 GEMM on the same weights dequantised beforehand
     pm = 1024
     per_shape, tot_flops, tot_sec = {}, 0.0, 0.0
     lib_shape, lib_sec = {}, 0.0
-    for name, k, n in LLAMA_DECODE:
+    for name, k, n in (LLAMA_DECODE if "prefill" in want else []):
         layer = Layer(name, k, n, pm, 2, dev, gen)
         sec, _ = time_graphs(lambda i: layer.run(i), 2, 100, 40)
         fl = linear_flops(pm, k, n)
@@ -600,27 +612,34 @@ def main():
         lib_sec += sec_l
         del layer, dense
         torch.cuda.empty_cache()
-    result["prefill_gemm_m1024"] = {
-        "metric": "W4A16 prefill GEMM TFLOP/s at M=1024 (same four linears)", "value": round(tot_flops / tot_sec / 1e12, 1),
-        "unit": "TFLOP/s", "us_per_layer": round(tot_sec * 1e6, 2), "per_linear": per_shape,
-        "roofline": {"bound": "mfma", "achieved": round(tot_flops / tot_sec / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
-                     "unit": "TFLOP/s", "frac": round(tot_flops / tot_sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
-                     "kernel": "w4a16_wide_kernel (256 x 256 tiles) for gate_up, w4a16_tile_kernel<MT> (MT = 4, or 2 for the "
-                               "6144-wide qkv) for the other three"}}
-    result["library_fp16_gemm_m1024"] = {
-        "what": "torch.matmul(x[1024, k] fp16, w[k, n] fp16) on the same weights dequantised beforehand (its dequantisation "
-                "pass not counted), same graph timing",
-        "value": round(tot_flops / lib_sec / 1e12, 1), "unit": "TFLOP/s", "us_per_layer": round(lib_sec * 1e6, 2),
-        "frac_of_peak": round(tot_flops / lib_sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4), "per_linear": lib_shape}
-    result["mfma_only_loop"] = mfma_loop(dev, gen)
-    # [us, fraction of the dense fp16 MFMA peak]
-    result["prefill_sweep"] = table(LLAMA_DECODE, (256, 4096))
-    # configs[3]: structured-pruned Llama (widths padded to multiples of 256 as the module pads them);
-    # down_proj behind the fused 128-block rotation.  configs[4]: the Mamba2 block.
-    result["pruned_llama"] = table(PRUNED, (1, 1024))
-    result["mamba2"] = table(MAMBA, (1, 1024))
-    result["mamba2"]["embedding_256000x4096_2048ids"] = embedding_gather(dev, gen)
-    result["secondary_kernels"] = secondary(dev, gen)
+    if "prefill" in want:
+        result["prefill_gemm_m1024"] = {
+            "metric": "W4A16 prefill GEMM TFLOP/s at M=1024 (same four linears)",
+            "value": round(tot_flops / tot_sec / 1e12, 1),
+            "unit": "TFLOP/s", "us_per_layer": round(tot_sec * 1e6, 2), "per_linear": per_shape,
+            "roofline": {"bound": "mfma", "achieved": round(tot_flops / tot_sec / 1e12, 1), "peak": MFMA_F16_PEAK_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(tot_flops / tot_sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                         "kernel": "w4a16_wide_kernel (256 x 256 tiles) for gate_up, w4a16_tile_kernel<MT> (MT = 4, or 2 "
+                                   "for the 6144-wide qkv) for the other three"}}
+        result["library_fp16_gemm_m1024"] = {
+            "what": "torch.matmul(x[1024, k] fp16, w[k, n] fp16) on the same weights dequantised beforehand (its "
+                    "dequantisation pass not counted), same graph timing",
+            "value": round(tot_flops / lib_sec / 1e12, 1), "unit": "TFLOP/s", "us_per_layer": round(lib_sec * 1e6, 2),
+            "frac_of_peak": round(tot_flops / lib_sec / 1e12 / MFMA_F16_PEAK_TFLOPS, 4), "per_linear": lib_shape}
+        result["mfma_only_loop"] = mfma_loop(dev, gen)
+    if "prefill_sweep" in want:
+        # [us, fraction of the dense fp16 MFMA peak]
+        result["prefill_sweep"] = table(LLAMA_DECODE, (256, 4096))
+    if "models" in want:
+        # configs[3]: structured-pruned Llama (widths padded to multiples of 256 as the module pads them);
+        # down_proj behind the fused 128-block rotation.  configs[4]: the Mamba2 block.
+        result["pruned_llama"] = table(PRUNED, (1, 1024))
+        result["mamba2"] = table(MAMBA, (1, 1024))
+        result["mamba2"]["embedding_256000x4096_2048ids"] = embedding_gather(dev, gen)
+    if "secondary" in want:
+        result["secondary_kernels"] = secondary(dev, gen)
+        if "models" not in want:
+            result["secondary_kernels"]["embedding_256000x4096_2048ids"] = embedding_gather(dev, gen)
     if args.sweep:
         sweep(dev, gen, args.sweep_json)
     if not args.no_cpu:
