@@ -33,6 +33,27 @@ def test_embedding_bit_exact(gpu, v, d, shape):
     assert np.array_equal(out.cpu().numpy().view(np.uint16), want.view(np.uint16))
 
 
+def test_embedding_scale_of_every_row_incl_the_last_of_an_odd_table(gpu):
+    """The kernel reads a row's 16-bit scale as half of an aligned 32-bit word where that word lies
+    inside the array, and as 16 bits otherwise: every id of an odd-sized and an even-sized table
+    (the last row of the odd one has no such word), and a scales tensor that starts at an odd
+    element of its storage (no 4-byte alignment)."""
+    from uniql_amd import ops
+    for v in (7, 8):
+        packed, scales = make_table(v, 64, 40 + v)
+        ids = np.arange(v, dtype=np.int64)
+        want = O.embedding_lookup(ids, packed, scales)
+        w = torch.from_numpy(packed).to(gpu)
+        out = ops.w4a16_embedding_lookup(torch.from_numpy(ids).to(gpu), w, torch.from_numpy(scales).to(gpu))
+        assert np.array_equal(out.cpu().numpy().view(np.uint16), want.view(np.uint16))
+        shifted = torch.zeros(v + 1, dtype=torch.float16, device=gpu)
+        shifted[1:] = torch.from_numpy(scales).to(gpu)
+        view = shifted[1:]
+        assert view.data_ptr() % 4 == 2
+        out = ops.w4a16_embedding_lookup(torch.from_numpy(ids).to(gpu), w, view)
+        assert np.array_equal(out.cpu().numpy().view(np.uint16), want.view(np.uint16))
+
+
 def test_embedding_module_from_fp16(gpu):
     from uniql_amd.quantize.quant_embedding_layers import W4O16Embedding
     g = torch.Generator().manual_seed(3)

@@ -115,62 +115,103 @@ __global__ __launch_bounds__(256) void rope_indices_lds_kernel(const RopeArgs a,
     typedef typename HalfVec<VEC>::type vec_t;
     extern __shared__ __attribute__((aligned(16))) uint32_t rope_lds[];
     uint16_t* trow = reinterpret_cast<uint16_t*>(rope_lds);  // the token's cos row, then its sin row
-    uint32_t* tab = rope_lds + ((cos_dim + 3) & ~3);         // entry (kv head, column): cos | sin << 16
+    // gathered tables: entry (kv head, column) of the cosines, then the same of the sines, as fp16
+    uint16_t* tab_cos = reinterpret_cast<uint16_t*>(rope_lds + ((cos_dim + 3) & ~3));
+    uint16_t* tab_sin = tab_cos + a.n_kh * a.hd;
     const int tid = threadIdx.x;
     const int64_t row = blockIdx.x;
     const int64_t table_row = a.cos_batch == 1 ? row % a.seq_len : row;
     const uint16_t* cos_row = reinterpret_cast<const uint16_t*>(a.cos + table_row * a.cos_row_stride);
     const uint16_t* sin_row = reinterpret_cast<const uint16_t*>(a.sin + table_row * a.cos_row_stride);
+    // Everything the token needs from memory is requested before the first barrier: the (cos, sin)
+    // row, the thread's first four index entries and its first two work items' q / k values are three
+    // independent loads, and issued one behind a barrier behind the other they would cost three
+    // memory round trips in a launch that lasts little longer than that.
+    const int entries = a.n_kh * a.hd;
+    const int half = a.hd >> 1;
+    const int per_head = half / VEC;
+    const int per_row = (a.n_qh + a.n_kh) * per_head;
+    constexpr int kIdxAhead = 4;
+    int idx_ahead[kIdxAhead];
+#pragma unroll
+    for (int i = 0; i < kIdxAhead; ++i) {
+        const int e = tid + 256 * i;
+        idx_ahead[i] = e < entries ? load_index(a.indices, a.index_bytes, e) : 0;
+    }
+    auto item = [&](int t, half_t*& x, int& kv_head, int& j) __attribute__((always_inline)) {
+        const int head = t / per_head;
+        j = (t - head * per_head) * VEC;
+        const bool is_q = head < a.n_qh;
+        kv_head = is_q ? head / (a.n_qh / a.n_kh) : head - a.n_qh;
+        x = is_q ? a.q + row * a.q_row_stride + (int64_t)head * a.hd
+                 : a.k + row * a.k_row_stride + (int64_t)(head - a.n_qh) * a.hd;
+    };
+    constexpr int kItemsAhead = 2;  // 32 + 8 heads of 128 are 320 work items of eight column pairs: two per thread at most
+    half_t* x0[kItemsAhead];
+    int kv0[kItemsAhead], j0[kItemsAhead];
+    vec_t lo0[kItemsAhead], hi0[kItemsAhead];
+#pragma unroll
+    for (int i = 0; i < kItemsAhead; ++i) {
+        x0[i] = nullptr;
+        kv0[i] = j0[i] = 0;
+        lo0[i] = hi0[i] = vec_t();
+        if (tid + 256 * i < per_row) {
+            item(tid + 256 * i, x0[i], kv0[i], j0[i]);
+            lo0[i] = *reinterpret_cast<const vec_t*>(x0[i] + j0[i]);
+            hi0[i] = *reinterpret_cast<const vec_t*>(x0[i] + half + j0[i]);
+        }
+    }
     for (int i = tid; i < cos_dim; i += 256) {
         trow[i] = cos_row[i];
         trow[cos_dim + i] = sin_row[i];
     }
     __syncthreads();
-    const int entries = a.n_kh * a.hd;
-    for (int e = tid; e < entries; e += 256) {
+#pragma unroll
+    for (int i = 0; i < kIdxAhead; ++i) {
+        const int e = tid + 256 * i;
+        if (e < entries) {
+            tab_cos[e] = trow[idx_ahead[i]];
+            tab_sin[e] = trow[cos_dim + idx_ahead[i]];
+        }
+    }
+    for (int e = tid + 256 * kIdxAhead; e < entries; e += 256) {
         const int i = load_index(a.indices, a.index_bytes, e);
-        tab[e] = (uint32_t)trow[i] | ((uint32_t)trow[cos_dim + i] << 16);
+        tab_cos[e] = trow[i];
+        tab_sin[e] = trow[cos_dim + i];
     }
     __syncthreads();
-    const int half = a.hd >> 1;
-    const int per_head = half / VEC;
-    const int per_row = (a.n_qh + a.n_kh) * per_head;
-    for (int t = tid; t < per_row; t += 256) {
-        const int head = t / per_head;
-        const int j = (t - head * per_head) * VEC;
-        const bool is_q = head < a.n_qh;
-        const int kv_head = is_q ? head / (a.n_qh / a.n_kh) : head - a.n_qh;
-        half_t* x = is_q ? a.q + row * a.q_row_stride + (int64_t)head * a.hd
-                         : a.k + row * a.k_row_stride + (int64_t)(head - a.n_qh) * a.hd;
-        vec_t lo_v = *reinterpret_cast<const vec_t*>(x + j), hi_v = *reinterpret_cast<const vec_t*>(x + half + j);
-        const uint32_t* e_lo = tab + kv_head * a.hd + j;
-        const uint32_t* e_hi = e_lo + half;
-#pragma unroll
-        for (int v = 0; v < VEC; ++v) {
-            const uint32_t w_lo = e_lo[v], w_hi = e_hi[v];
-            const half_t c_lo = __builtin_bit_cast(half_t, (uint16_t)(w_lo & 0xffffu));
-            const half_t s_lo = __builtin_bit_cast(half_t, (uint16_t)(w_lo >> 16));
-            const half_t c_hi = __builtin_bit_cast(half_t, (uint16_t)(w_hi & 0xffffu));
-            const half_t s_hi = __builtin_bit_cast(half_t, (uint16_t)(w_hi >> 16));
-            half_t lo, hi;
-            if constexpr (VEC == 1) {
-                lo = lo_v;
-                hi = hi_v;
-            } else {
-                lo = lo_v[v];
-                hi = hi_v[v];
-            }
-            rotate_pair(lo, hi, c_lo, s_lo, c_hi, s_hi);
-            if constexpr (VEC == 1) {
-                lo_v = lo;
-                hi_v = hi;
-            } else {
-                lo_v[v] = lo;
-                hi_v[v] = hi;
-            }
+    auto rotate_item = [&](half_t* x, int kv_head, int j, vec_t lo_v, vec_t hi_v) __attribute__((always_inline)) {
+        const int e0 = kv_head * a.hd + j;
+        if constexpr (VEC > 1) {
+            // All of the item's column pairs at once in packed fp16 arithmetic.  An fp16 product or sum
+            // computed in fp32 and rounded to fp16 equals the fp16 operation's own single rounding
+            // (fp32's 24 bits are at least 2 x 11 + 2), so these are the values of rotate_pair bit for
+            // bit, at a fifth of its instructions: the conversions made this kernel compute-bound.
+#pragma clang fp contract(off)
+            const vec_t c_lo = *reinterpret_cast<const vec_t*>(tab_cos + e0), s_lo = *reinterpret_cast<const vec_t*>(tab_sin + e0);
+            const vec_t c_hi = *reinterpret_cast<const vec_t*>(tab_cos + e0 + half);
+            const vec_t s_hi = *reinterpret_cast<const vec_t*>(tab_sin + e0 + half);
+            const vec_t a_lo = lo_v * c_lo, r_lo = (-hi_v) * s_lo;
+            const vec_t a_hi = hi_v * c_hi, r_hi = lo_v * s_hi;
+            *reinterpret_cast<vec_t*>(x + j) = a_lo + r_lo;
+            *reinterpret_cast<vec_t*>(x + half + j) = a_hi + r_hi;
+        } else {
+            half_t lo = lo_v, hi = hi_v;
+            rotate_pair(lo, hi, __builtin_bit_cast(half_t, tab_cos[e0]), __builtin_bit_cast(half_t, tab_sin[e0]),
+                        __builtin_bit_cast(half_t, tab_cos[e0 + half]), __builtin_bit_cast(half_t, tab_sin[e0 + half]));
+            *reinterpret_cast<vec_t*>(x + j) = lo;
+            *reinterpret_cast<vec_t*>(x + half + j) = hi;
         }
-        *reinterpret_cast<vec_t*>(x + j) = lo_v;
-        *reinterpret_cast<vec_t*>(x + half + j) = hi_v;
+    };
+#pragma unroll
+    for (int i = 0; i < kItemsAhead; ++i)
+        if (tid + 256 * i < per_row) rotate_item(x0[i], kv0[i], j0[i], lo0[i], hi0[i]);
+    for (int t = tid + 256 * kItemsAhead; t < per_row; t += 256) {
+        half_t* x;
+        int kv_head, j;
+        item(t, x, kv_head, j);
+        const vec_t lo_v = *reinterpret_cast<const vec_t*>(x + j), hi_v = *reinterpret_cast<const vec_t*>(x + half + j);
+        rotate_item(x, kv_head, j, lo_v, hi_v);
     }
 }
 
