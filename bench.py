@@ -530,7 +530,7 @@ def main():
                    "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "wall_ms_per_step": round(wall_per_step * 1e3, 6)},
         "roofline": {"bound": "hbm", "achieved": round(gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
-                     "kernel": "w4a16_stream_kernel<RC=1, HAD=0, WAVES=4, EXT=false> (all four launches of a step)",
+                     "kernel": "w4a16_stream_kernel<RC=1, HAD=0, WAVES, EXT=false> (all four launches of a step; WAVES = 8 for down_proj, 4 for the others)",
                      "launches_per_step": launches,
                      "avg_launch_us": round(kernel_us, 3), "bytes_per_launch": step_bytes // launches},
     }

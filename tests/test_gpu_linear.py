@@ -82,6 +82,67 @@ def test_stream_kernel_llama_shapes(gpu, m, k, n):
     check_layer_output(y16, ref)
 
 
+def _scales_across_the_expansion_ranges(groups, n, seed):
+    """Scales inside the range of the streaming kernel's short expansion (2^-10 <= s < 2^-4, every
+    binade, both ends), and outside it on every side: zero, subnormal, just below 2^-10, 2^-4 and
+    above, large, negative."""
+    rng = np.random.default_rng(seed)
+    inside = np.concatenate([
+        np.array([2.0 ** -10, 2.0 ** -4 - 2.0 ** -15, 0.004, 0.02, 0.0624], dtype=np.float16),
+        (2.0 ** rng.uniform(-10, -4, size=64)).astype(np.float16)])
+    inside = inside[(inside >= np.float16(2.0 ** -10)) & (inside < np.float16(2.0 ** -4))]
+    outside = np.array([0.0, 6e-8, 2.0 ** -14, np.nextafter(np.float16(2.0 ** -10), np.float16(0)), 2.0 ** -4, 0.07,
+                        0.5, 3.0, 1000.0, -0.01, -2.0 ** -12], dtype=np.float16)
+    s = rng.choice(inside, size=(groups, n)).astype(np.float16)
+    return s, outside, rng
+
+
+def test_stream_kernel_reproduces_every_weight(gpu):
+    """One-hot activation rows make every output element a single product 1 * w, exact in the
+    matrix unit and in fp32: the streaming kernel's fp32 output must then BE the reference's
+    fp16 weight fp16_rn((code - 8) * scale) (marlin_gemm_kernel.cuh:118-146), for all 16 codes,
+    for scales over the whole range of the short expansion (both code positions of a packed
+    word: the low one is held divided by 16 and multiplied back at the end) and for scales
+    outside it, which take the long expansion (a wave switches when any of its lanes meets one)."""
+    k, n, groups = 256, 256, 2
+    s, outside, rng = _scales_across_the_expansion_ranges(groups, n, 11)
+    # group 0: every column in range; group 1: out-of-range scales in a third of the columns
+    cols = rng.choice(n, size=n // 3, replace=False)
+    s[1, cols] = rng.choice(outside, size=cols.size)
+    q = rng.integers(0, 16, size=(k, n)).astype(np.int32)
+    q[:16] = np.arange(16)[:, None]          # every code in every column at least once per class of K row
+    q[16:32] = np.arange(16)[::-1, None]
+    w = O.dequant_codes(q, s, 128)
+    p = dict(q=q, s=s, m=16, k=k, n=n, packed=O.pack_weights(q), s_perm=O.permute_scales(s, k, n, 128))
+    for k0 in range(0, k, 16):
+        x = np.zeros((16, k), dtype=np.float16)
+        x[np.arange(16), k0 + np.arange(16)] = 1.0
+        p["x"] = x
+        y32 = run_gemm(p, gpu, out_f32=True)
+        want = w[k0:k0 + 16].astype(np.float32)
+        assert np.array_equal(y32, want), (k0, np.abs(y32 - want).max())
+
+
+@pytest.mark.parametrize("m", [1, 6])
+def test_scales_outside_the_short_expansion_range(gpu, m):
+    """Random data with out-of-range scales sprinkled over groups and columns (so that some waves
+    switch between the two expansions from one group to the next), with and without a K split."""
+    k, n = 2048, 512
+    p = make_linear_problem(m, k, n, seed=400 + m)
+    s, outside, rng = _scales_across_the_expansion_ranges(k // 128, n, 12 + m)
+    hit = rng.random(s.shape) < 0.02
+    s[hit] = rng.choice(outside[np.abs(outside) <= 3.0], size=int(hit.sum()))
+    s[5, :] = np.float16(0.25)               # a whole group outside
+    p["s"] = s
+    p["s_perm"] = O.permute_scales(s, k, n, 128)
+    w = O.dequant_codes(p["q"], s, 128)
+    ref = O.gemm_fp64(p["x"], w)
+    budget = np.abs(p["x"].astype(np.float64)) @ np.abs(w.astype(np.float64))   # sum of |terms| per output
+    for flags in (0, (8 << 8) | (4 << 16)):   # the default plan (K split) and one workgroup per strip
+        y32 = run_gemm(p, gpu, out_f32=True, flags=flags)
+        assert (np.abs(y32 - ref) <= 2.0 ** -20 * budget + 1e-30).all(), np.abs(y32 - ref).max()
+
+
 F_FORCE_SKINNY, F_FORCE_TILED = 2, 4
 
 

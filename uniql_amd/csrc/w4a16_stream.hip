@@ -16,15 +16,20 @@
 // M = 1..16 all run at the weight-streaming rate.
 //
 // Every weight is expanded to the reference's fp16 value fp16_rn((code - 8) * scale)
-// (csrc/linear/marlin_gemm_kernel.cuh:118-146) before it enters the matrix unit: 13 vector
-// instructions per packed word (one shift, four mask-and-or, two fp16 subtractions, two fp16
-// fused multiply-adds, four fp16 multiplications by the scale), all exact except the final
-// multiplication, which rounds once as the reference's does.  The products are exact in the
-// MFMA and accumulate in fp32, so the result equals the reference's value up to the order of
-// the fp32 additions, for every M.  (Feeding the raw codes as fp16 subnormals and scaling each
-// group's fp32 dot product instead saves 8 of the 13 instructions, but leaves out the fp16
-// rounding of the scaled weights: up to 5e-3 away from the reference's value at K = 14336,
-// which an fp16 output between 16 and 32 cannot absorb inside a max-abs tolerance of 1e-2.)
+// (csrc/linear/marlin_gemm_kernel.cuh:118-146) before it enters the matrix unit; the products are
+// exact in the MFMA and accumulate in fp32, so the result equals the reference's value up to the
+// order of the fp32 additions, for every M.  Two expansions give that value (see process()):
+//   * short, 9 vector instructions per packed word (a shift, four ANDs, four fused multiply-adds
+//     whose first operand is the masked code read as an fp16 subnormal), exact while every scale of
+//     the wave's unit lies in [2^-10, 2^-4); the weights from the low code position come out
+//     divided by 16 and are summed apart;
+//   * long, 13 instructions (a shift, four mask-and-or into [1024, 1040), two subtractions, two
+//     fused multiply-adds, four multiplications by the scale), exact for every scale; a wave takes
+//     it for a unit in which any lane's check of its scales fails.
+// (Feeding the raw codes to the matrix unit and scaling each group's fp32 dot product instead
+// would need 5 instructions, but leaves out the fp16 rounding of the scaled weights: up to 5e-3
+// away from the reference's value at K = 14336, which an fp16 output between 16 and 32 cannot
+// absorb inside a max-abs tolerance of 1e-2.)
 //
 // Work split: unit = (strip of 128 columns) x (group of 128 K).  A wave owns `upw`
 // consecutive groups of a strip, the four or eight waves of a workgroup own consecutive
@@ -108,19 +113,22 @@ void w4a16_stream_kernel(const StreamArgs a) {
     const u32x4* strip_w = a.B + (size_t)strip * 64;
     const half_t* strip_s = a.S + (size_t)strip * 128;
 
-    f4 acc[8];  // acc[jb][v]: output row 4 kq + v, column slot jb of this lane
+    // acc[jb][v]: output row 4 kq + v, column slot jb of this lane; acc_low collects the products of
+    // the weights that the short expansion leaves divided by 16 (see process)
+    f4 acc[8], acc_low[8];
 #pragma unroll
-    for (int jb = 0; jb < 8; ++jb) acc[jb] = f4{0.f, 0.f, 0.f, 0.f};
+    for (int jb = 0; jb < 8; ++jb) acc[jb] = acc_low[jb] = f4{0.f, 0.f, 0.f, 0.f};
 
     uint32_t* xs = lds + (size_t)w * a.xrows * kXsStride;  // this wave's staging rows
-    // Staged row layout (dwords): the pair of K values 2d, 2d+1 of the group, d = 16 rp + kq' + 4 t,
-    // sits at dword 16 rp + 4 kq' + t, so that the A operand of lane (row, kq') for row pair rp
-    // is one 16-byte read.
+    // Staged row layout (dwords): the pair of K values 2d, 2d+1 of the group, d = 32 rq + 8 i + kq' + 4 c
+    // (packed row 4 rq + i of the group, K rows 2 kq', 2 kq' + 1 for c = 0 or 2 kq' + 8, 2 kq' + 9 for
+    // c = 1), sits at dword 32 rq + 16 c + 4 kq' + i, so that the A operand of lane (row, kq') for
+    // the low (c = 0) or high (c = 1) code pairs of the four packed rows of quad rq is one 16-byte read.
     // MFMA row `slot` reads staged row min(slot, xrows - 1): rows past M only feed output rows
     // that are never stored.
     const int xrow_of = (slot < a.xrows ? slot : a.xrows - 1) * kXsStride + 4 * kq;
-    // where this lane's staged quad goes: lane `slot` holds pairs d = 4 slot + i
-    const int stage_off = 16 * (slot >> 2) + (slot & 3);
+    // where this lane's staged quad goes: lane `slot` holds pairs d = 4 slot + p, written 4 p apart
+    const int stage_off = 32 * (slot >> 3) + 16 * (slot & 1) + ((slot & 7) >> 1);
     NibbleMagic magic;
     magic.init();
 
@@ -220,27 +228,96 @@ void w4a16_stream_kernel(const StreamArgs a) {
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 
-        // Row pair rp (packed rows 2rp, 2rp+1 = 32 K values) against the eight column slots
-        // jb = 2j + blk of this lane: the B operand is the four code pairs of words j of both
-        // packed rows (low byte pair for blk 0, after >> 8 for blk 1), expanded and scaled; the
-        // scale of column slot jb is half jb of the 16-byte scale load.  Consecutive MFMAs go to
-        // different accumulators.
+        // Quad rq (packed rows 4 rq .. 4 rq + 3 = 64 K values) against the eight column slots
+        // jb = 2 j + blk of this lane.  Word j of a packed row holds, for blk 0 and (after >> 8) for
+        // blk 1, a LOW code pair (bits 0..3 and 16..19: K rows 2 kq, 2 kq + 1) and a HIGH code pair
+        // (bits 4..7 and 20..23: K rows 2 kq + 8, 2 kq + 9).  One MFMA takes the low pairs of the
+        // quad's four rows, the next the high pairs; the scale of column slot jb is half jb of the
+        // 16-byte scale load.
+        //
+        // Short expansion.  A code c left where it is, everything else masked away, IS an fp16
+        // number: c 2^-20 in the high position, c 2^-24 in the low one (subnormals, exact).  With
+        // S = s 2^20 one fused multiply-add gives
+        //     high:  fma(c 2^-20, S, -8 s)  = fp16_rn((c - 8) s)
+        //     low:   fma(c 2^-24, S, -s/2)  = fp16_rn((c - 8) s / 16) = fp16_rn((c - 8) s) / 16
+        // exactly (one rounding of the exact value, as the reference's multiplication makes), PROVIDED
+        // S, 8 s and s / 2 are exact and the low form's result is a normal number whenever it is not
+        // zero: 2^-10 <= s < 2^-4.  The low pairs' products are summed apart (acc_low) and enter the
+        // result times 16 at the end: a power of two, exact in fp32.  9 vector instructions per packed
+        // word (a shift, four ANDs, four FMAs) instead of 13.  A lane checks its eight scales; if any
+        // lane of the wave finds one outside the range (or zero: padding columns, empty groups), the
+        // whole wave expands this unit the long way (mask-and-or into [1024, 1040), subtract, multiply:
+        // exact for every scale), into the same accumulators.
+        // range check on both halves of a scale word at once: t = bits - 0x1400 must lie below 0x1800,
+        // i.e. neither t nor t + 0x0800 may have one of its three top bits set (a borrow or carry
+        // between the halves only happens next to a half that fails anyway)
+        uint32_t out_of_range = 0;
 #pragma unroll
-        for (int rp = 0; rp < RPW; ++rp) {
-            const h8 xa = __builtin_bit_cast(h8, *reinterpret_cast<const u32x4*>(xs + xrow_of + 16 * rp));
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t t = scales[j] - 0x14001400u;
+            out_of_range |= t | (t + 0x08000800u);
+        }
+        const bool lane_ok = (out_of_range & 0xE000E000u) == 0;
+        if (__builtin_expect(__builtin_amdgcn_ballot_w64(!lane_ok) == 0ull, 1)) {
+            h2 s20[4], c_high[4], c_low[4];
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const uint32_t q0 = r.wq[2 * rp][j], q1 = r.wq[2 * rp + 1][j];
                 const h2 pr = bits_to_h2(scales[j]);
+                s20[j] = bits_to_h2(scales[j] + 0x50005000u);  // exponents + 20 (both are normal and stay in range)
+                c_high[j] = pr * h2{(half_t)-8.0f, (half_t)-8.0f};
+                c_low[j] = pr * h2{(half_t)-0.5f, (half_t)-0.5f};
+            }
 #pragma unroll
-                for (int blk = 0; blk < 2; ++blk) {
-                    const uint32_t p0 = blk ? (q0 >> 8) : q0;
-                    const uint32_t p1 = blk ? (q1 >> 8) : q1;
-                    const h2 sv = blk ? h2{pr.y, pr.y} : h2{pr.x, pr.x};
-                    const h2 e0 = magic.pair_low(p0) * sv, e1 = magic.pair_high(p0) * sv;
-                    const h2 e2 = magic.pair_low(p1) * sv, e3 = magic.pair_high(p1) * sv;
-                    const h8 bw = h8{e0.x, e0.y, e1.x, e1.y, e2.x, e2.y, e3.x, e3.y};
-                    acc[2 * j + blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa, bw, acc[2 * j + blk], 0, 0, 0);
+            for (int rq = 0; rq < RPW / 2; ++rq) {
+                const h8 xa_low = __builtin_bit_cast(h8, *reinterpret_cast<const u32x4*>(xs + xrow_of + 32 * rq));
+                const h8 xa_high = __builtin_bit_cast(h8, *reinterpret_cast<const u32x4*>(xs + xrow_of + 32 * rq + 16));
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+#pragma unroll
+                    for (int blk = 0; blk < 2; ++blk) {
+                        const h2 sv = blk ? h2{s20[j].y, s20[j].y} : h2{s20[j].x, s20[j].x};
+                        const h2 ch = blk ? h2{c_high[j].y, c_high[j].y} : h2{c_high[j].x, c_high[j].x};
+                        const h2 cl = blk ? h2{c_low[j].y, c_low[j].y} : h2{c_low[j].x, c_low[j].x};
+                        h2 el[4], eh[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const uint32_t q = r.wq[4 * rq + i][j];
+                            const uint32_t pq = blk ? (q >> 8) : q;
+                            el[i] = __builtin_elementwise_fma(bits_to_h2(pq & magic.mask_low), sv, cl);
+                            eh[i] = __builtin_elementwise_fma(bits_to_h2(pq & magic.mask_high), sv, ch);
+                        }
+                        const h8 bl = h8{el[0].x, el[0].y, el[1].x, el[1].y, el[2].x, el[2].y, el[3].x, el[3].y};
+                        const h8 bh = h8{eh[0].x, eh[0].y, eh[1].x, eh[1].y, eh[2].x, eh[2].y, eh[3].x, eh[3].y};
+                        acc_low[2 * j + blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa_low, bl, acc_low[2 * j + blk], 0, 0, 0);
+                        acc[2 * j + blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa_high, bh, acc[2 * j + blk], 0, 0, 0);
+                        
+                    }
+                }
+            }
+        } else {
+#pragma unroll
+            for (int rq = 0; rq < RPW / 2; ++rq) {
+                const h8 xa_low = __builtin_bit_cast(h8, *reinterpret_cast<const u32x4*>(xs + xrow_of + 32 * rq));
+                const h8 xa_high = __builtin_bit_cast(h8, *reinterpret_cast<const u32x4*>(xs + xrow_of + 32 * rq + 16));
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const h2 pr = bits_to_h2(scales[j]);
+#pragma unroll
+                    for (int blk = 0; blk < 2; ++blk) {
+                        const h2 sv = blk ? h2{pr.y, pr.y} : h2{pr.x, pr.x};
+                        h2 el[4], eh[4];
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const uint32_t q = r.wq[4 * rq + i][j];
+                            const uint32_t pq = blk ? (q >> 8) : q;
+                            el[i] = magic.pair_low(pq) * sv;
+                            eh[i] = magic.pair_high(pq) * sv;
+                        }
+                        const h8 bl = h8{el[0].x, el[0].y, el[1].x, el[1].y, el[2].x, el[2].y, el[3].x, el[3].y};
+                        const h8 bh = h8{eh[0].x, eh[0].y, eh[1].x, eh[1].y, eh[2].x, eh[2].y, eh[3].x, eh[3].y};
+                        acc[2 * j + blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa_low, bl, acc[2 * j + blk], 0, 0, 0);
+                        acc[2 * j + blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa_high, bh, acc[2 * j + blk], 0, 0, 0);
+                    }
                 }
             }
         }
@@ -277,6 +354,8 @@ void w4a16_stream_kernel(const StreamArgs a) {
     if (HAD == 2)  // all waves, also those without groups: the transform has workgroup barriers
         fwht_rows_to_lds<kRowChunks>(xin, reinterpret_cast<float*>(lds + a.fwht_lds), a.M, a.K, a.log2K, tid, 64 * WAVES);
     auto finish = [&]() __attribute__((always_inline)) {
+#pragma unroll
+    for (int jb = 0; jb < 8; ++jb) acc[jb] += acc_low[jb] * 16.0f;
     // ---- combine the waves (fixed order), then the K splits ------------------------------
     // acc[jb][v] on lane l is row m = 4 (l/16) + v, column
     // 128 strip + 64 (slot/8) + 16 (jb/2) + 8 (jb%2) + slot%8.
@@ -400,18 +479,20 @@ struct StreamPlan {
 
 // Heuristic (from sweeps over waves x groups per wave on the Llama, pruned-Llama and Mamba2 shapes
 // at 1, 2, 4 and 8 rows):
-//   * enough strips to occupy the chip on their own (>= 176): one workgroup owns a whole strip, so
-//     no partial sums are exchanged between workgroups; four waves with eight groups each when K
-//     allows it (long streams per wave, two register sets in flight), else eight waves;
-//   * otherwise K is split over workgroups.  One or two rows: 4 waves, and as many groups per wave
-//     as it takes to stay within about 288 workgroups.  More rows: every split costs a 64-bit
-//     atomic per output element, so 8 waves (4 for small problems: below 1536 units, from 8 rows on
-//     below 768) and at most 256 workgroups.
+//   * enough strips to occupy most of the chip on their own (>= 144): one workgroup owns a whole
+//     strip, so no partial sums are exchanged between workgroups; four waves with eight groups each
+//     when K allows it (long streams per wave, two register sets in flight), else eight waves;
+//   * otherwise K is split over workgroups.  One or two rows: as many groups per workgroup as it
+//     takes to stay within about 288 workgroups, on 4 waves, or, from four groups per wave on, on 8
+//     waves with half as many each (two waves per SIMD cover each other's waits: 14336 -> 4096 at
+//     one row 8.2 against 8.6 us).  More rows: every split costs a 64-bit atomic per output element,
+//     so 8 waves (4 for small problems: below 1536 units, from 8 rows on below 768) and at most 256
+//     workgroups.
 static StreamPlan stream_plan(int m, int n, int k, int upw_override, int waves_override) {
     const int nstrips = n / 128, G = k / 128;
     const int64_t units = (int64_t)nstrips * G;
     StreamPlan p;
-    const bool whole_strip = m <= 16 && nstrips >= 176 && G >= 16 && G <= 64;
+    const bool whole_strip = m <= 16 && nstrips >= 144 && G >= 16 && G <= 64;
     int max_wgs = 288;
     if (waves_override) {
         p.waves = waves_override;
@@ -430,10 +511,10 @@ static StreamPlan stream_plan(int m, int n, int k, int upw_override, int waves_o
     } else {
         p.upw = 1;
         while (p.upw < 8 && (int64_t)nstrips * ceil_div(G, p.waves * p.upw) > max_wgs) ++p.upw;
-        // one or two rows and a strip count that lands well below the chip's 256 compute units once
-        // the grid is inside the limit (146 strips: 292 workgroups are too many, 146 too few): one
-        // group per wave and many short workgroups instead (4096 -> 18688 at one row: 10.5 against 11.3 us)
-        if (m <= 2 && p.upw > 1 && (int64_t)nstrips * ceil_div(G, p.waves * p.upw) < 176) p.upw = 1;
+        if (m <= 2 && !waves_override && p.waves == 4 && p.upw >= 4 && p.upw % 2 == 0) {
+            p.waves = 8;
+            p.upw /= 2;
+        }
     }
     p.splits = ceil_div(G, p.waves * p.upw);
     while (p.splits > kAccumMaxSplits) {  // the contribution count has 7 bits
