@@ -143,6 +143,24 @@ def test_scales_outside_the_short_expansion_range(gpu, m):
         assert (np.abs(y32 - ref) <= 2.0 ** -20 * budget + 1e-30).all(), np.abs(y32 - ref).max()
 
 
+def test_per_column_scales_outside_the_short_expansion_range(gpu):
+    """One scale per column (a single scale row): a column outside the range sends its wave the long
+    way in every group; one-hot rows again make the output the weights themselves."""
+    k, n = 256, 256
+    s, outside, rng = _scales_across_the_expansion_ranges(1, n, 21)
+    cols = rng.choice(n, size=40, replace=False)
+    s[0, cols] = rng.choice(outside, size=cols.size)
+    q = rng.integers(0, 16, size=(k, n)).astype(np.int32)
+    w = O.dequant_codes(q, s, k)
+    p = dict(q=q, s=s, m=16, k=k, n=n, packed=O.pack_weights(q), s_perm=O.permute_scales(s, k, n, k))
+    for k0 in (0, 112, 240):
+        x = np.zeros((16, k), dtype=np.float16)
+        x[np.arange(16), k0 + np.arange(16)] = 1.0
+        p["x"] = x
+        y32 = run_gemm(p, gpu, out_f32=True)
+        assert np.array_equal(y32, w[k0:k0 + 16].astype(np.float32)), k0
+
+
 F_FORCE_SKINNY, F_FORCE_TILED = 2, 4
 
 
