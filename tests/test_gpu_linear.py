@@ -382,6 +382,24 @@ def test_fused_blockwise_hadamard(gpu, m):
     check_layer_output(run_gemm(p, gpu, had_block=128, had_scale=128 ** -0.5), ref)
 
 
+@pytest.mark.parametrize("had_block", [128, 2048])
+def test_rotations_with_scales_outside_the_short_expansion_range(gpu, had_block):
+    """The fused rotations (128-blocks while staging; whole rows in LDS) in front of units that
+    take the long expansion and units that take the short one."""
+    m, k, n = 3, 2048, 384
+    p = make_linear_problem(m, k, n, seed=had_block)
+    s, outside, rng = _scales_across_the_expansion_ranges(k // 128, n, had_block + 1)
+    hit = rng.random(s.shape) < 0.03
+    s[hit] = rng.choice(outside[np.abs(outside) <= 3.0], size=int(hit.sum()))
+    p["s"], p["s_perm"] = s, O.permute_scales(s, k, n, 128)
+    xr = O.fwht(p["x"], had_block ** -0.5, block=had_block)
+    w = O.dequant_codes(p["q"], s, 128)
+    ref = O.gemm_fp64(xr, w)
+    budget = np.abs(xr.astype(np.float64)) @ np.abs(w.astype(np.float64))
+    y32 = run_gemm(p, gpu, out_f32=True, had_block=had_block, had_scale=had_block ** -0.5)
+    assert (np.abs(y32 - ref) <= 2.0 ** -20 * budget + 1e-30).all(), np.abs(y32 - ref).max()
+
+
 @pytest.mark.parametrize("m", [1, 3])
 def test_full_width_hadamard_prologue(gpu, m):
     k, n = 8192, 256
