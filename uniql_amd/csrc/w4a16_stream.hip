@@ -248,7 +248,8 @@ void w4a16_stream_kernel(const StreamArgs a) {
         // lane of the wave finds one outside the range (or zero: padding columns, empty groups), the
         // whole wave expands this unit the long way (mask-and-or into [1024, 1040), subtract, multiply:
         // exact for every scale), into the same accumulators.
-        // range check on both halves of a scale word at once: t = bits - 0x1400 must lie below 0x1800,
+        //
+        // Range check on both halves of a scale word at once: t = bits - 0x1400 must lie below 0x1800,
         // i.e. neither t nor t + 0x0800 may have one of its three top bits set (a borrow or carry
         // between the halves only happens next to a half that fails anyway)
         uint32_t out_of_range = 0;
@@ -290,7 +291,6 @@ void w4a16_stream_kernel(const StreamArgs a) {
                         const h8 bh = h8{eh[0].x, eh[0].y, eh[1].x, eh[1].y, eh[2].x, eh[2].y, eh[3].x, eh[3].y};
                         acc_low[2 * j + blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa_low, bl, acc_low[2 * j + blk], 0, 0, 0);
                         acc[2 * j + blk] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa_high, bh, acc[2 * j + blk], 0, 0, 0);
-                        
                     }
                 }
             }
