@@ -9,8 +9,9 @@
 //     lane l :  slot = l % 16  ->  chunk = 2*strip + slot/8,  c8 = slot % 8
 //               kq   = l / 16  ->  piece 4*c8 + kq
 //
-// Every byte of the 1 KiB row segment is fetched once and eight MFMAs (one per jb)
-// consume two packed rows (32 K values) at a time.  The activations are the A operand:
+// Every byte of the 1 KiB row segment is fetched once and sixteen MFMAs (per jb one for the
+// low and one for the high code pairs of the words) consume four packed rows (64 K values) at
+// a time.  The activations are the A operand:
 // rows of X (up to 16 per launch) staged through LDS in the same K order.  MFMA is
 // used purely as a wide dot-product unit: its cost does not depend on M, so
 // M = 1..16 all run at the weight-streaming rate.
