@@ -9,7 +9,7 @@ LOW, HIGH = 0x1400, 0x2C00   # bit patterns of 2^-10 and 2^-4: the range is [LOW
 
 
 def fp16_fma(a, b, c):
-    with np.errstate(over="ignore"):   # scales past the range overflow on purpose (inf * 0 -> NaN is the point of one test)
+    with np.errstate(over="ignore", invalid="ignore"):   # scales past the range overflow on purpose (inf * 0 -> NaN is the point of one test)
         return (a.astype(np.float64) * b.astype(np.float64) + c.astype(np.float64)).astype(np.float16)
 
 
