@@ -357,6 +357,13 @@ void w4a16_stream_kernel(const StreamArgs a) {
     auto finish = [&]() __attribute__((always_inline)) {
 #pragma unroll
     for (int jb = 0; jb < 8; ++jb) acc[jb] += acc_low[jb] * 16.0f;
+    // The output stage's kernel arguments are fetched here, under the exchange of the partial sums
+    // (left to itself the compiler loads each of them in front of its first use: a scalar load and
+    // its wait in front of every row's atomic and again in front of its store).
+    const int n_splits = a.splits, n_cols = a.N, m_rows = a.M;
+    unsigned long long* const accum_base = a.accum;
+    void* const d_base = a.D;
+    asm volatile("" ::"s"(n_splits), "s"(n_cols), "s"(m_rows), "s"(accum_base), "s"(d_base));
     // ---- combine the waves (fixed order), then the K splits ------------------------------
     // acc[jb][v] on lane l is row m = 4 (l/16) + v, column
     // 128 strip + 64 (slot/8) + 16 (jb/2) + 8 (jb%2) + slot%8.
@@ -397,7 +404,7 @@ void w4a16_stream_kernel(const StreamArgs a) {
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
             const int ml = (tid >> 7) + RPT * i;
-            if (ml < a.M) {
+            if (ml < m_rows) {
 #pragma unroll
                 for (int ww = 0; ww < wpr; ++ww) {
                     tot[i] += red[(ww * rr_rows + ml) * 128 + col_out];
@@ -409,27 +416,27 @@ void w4a16_stream_kernel(const StreamArgs a) {
 #pragma unroll
     for (int i = 0; i < NI; ++i) {
         const int m = (tid >> 7) + RPT * i;
-        if (m >= a.M) continue;
-        unsigned long long* word = a.accum + (size_t)m * a.N + n_out;
+        if (m >= m_rows) continue;
+        unsigned long long* word = accum_base + (size_t)m * n_cols + n_out;
         if (!gated) {
             float total = tot[i];
-            const bool mine = a.splits == 1 || accum_add(word, tot[i], a.splits, total);
+            const bool mine = n_splits == 1 || accum_add(word, tot[i], n_splits, total);
             if (mine) {
                 if constexpr (EXT) {
-                    finish_store(a.epi, a.D, m, n_out, total);
+                    finish_store(a.epi, d_base, m, n_out, total);
                 } else {  // (fp32 output is one of the extended instantiation's cases)
-                    reinterpret_cast<half_t*>(a.D)[(size_t)m * a.N + n_out] = (half_t)total;
+                    reinterpret_cast<half_t*>(d_base)[(size_t)m * n_cols + n_out] = (half_t)total;
                 }
-                if (a.splits != 1) accum_reset(word);
+                if (n_splits != 1) accum_reset(word);
             }
         } else if (col_out < 64) {
             const int n_pair = 64 * strip + col_out;
-            if (a.splits == 1) {
-                finish_store_gated(a.epi, a.D, m, n_pair, tot[i], oth[i]);
+            if (n_splits == 1) {
+                finish_store_gated(a.epi, d_base, m, n_pair, tot[i], oth[i]);
             } else {
                 float total_g, total_u;
-                if (accum_add_pair(word, word + 64, tot[i], oth[i], a.splits, total_g, total_u)) {
-                    finish_store_gated(a.epi, a.D, m, n_pair, total_g, total_u);
+                if (accum_add_pair(word, word + 64, tot[i], oth[i], n_splits, total_g, total_u)) {
+                    finish_store_gated(a.epi, d_base, m, n_pair, total_g, total_u);
                     accum_reset(word);
                 }
             }
